@@ -4,8 +4,15 @@
 //                  the row's `top` largest logits at their places, zero elsewhere).  One wave per
 //                  row: each lane keeps E / 64 logits in registers, `top` rounds of a wave-wide
 //                  arg-max (ties: lowest index).
-//   sm_gated_act   act(gate) * up over stacked [gate | up] blocks (act: SiLU, ReLU or tanh-GELU),
-//                  expert e's block scaled by the row's routing weight; fp32 math.
+//   sm_route_groups  sigmoid router with a choice correction and a limit to the best groups of
+//                  experts: s = sigmoid(z), the choice ranks c = s + correction, a group of
+//                  neighbouring experts ranks by the sum of its largest c, only experts of the
+//                  `keep` best groups are eligible, the `top` eligible experts with the largest c
+//                  get s / (sum of the chosen s + eps) * scale.  One wave per row, the row's c in
+//                  LDS; every arg-max breaks ties towards the lowest index.
+//   sm_gated_act   act(gate) * up over stacked [gate | up] blocks (act: SiLU, ReLU, tanh-GELU or
+//                  squared ReLU), expert e's block scaled by the row's routing weight; fp32 math.
+//   sm_scaled_act  act(up) over stacked up blocks of experts without a gate, scaled the same way.
 //   sm_write_k     rows of the key projection into the paged key cache by slot.
 #include "seqmix.h"
 
@@ -15,9 +22,141 @@ namespace {
 
 constexpr int kMaxPerLane = 16;   // experts <= 1024
 
-// the gate's activation: 0 SiLU, 1 ReLU, 2 tanh-GELU
+// the gate's activation: 0 SiLU, 1 ReLU, 2 tanh-GELU, 3 squared ReLU
 __device__ __forceinline__ float gate_act(float g, int act) {
+  if (act == 3) {
+    const float r = fmaxf(g, 0.f);
+    return r * r;
+  }
   return act == 0 ? silu_f(g) : act == 1 ? fmaxf(g, 0.f) : gelu_tanh_f(g);
+}
+
+// wave-wide arg-max of (value, index) pairs, ties to the lowest index; every lane gets the result
+__device__ __forceinline__ void wave_argmax(float& bv, int& bi) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, 64);
+    const int oi = __shfl_xor(bi, o, 64);
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+  }
+}
+
+constexpr int kNone = 0x7fffffff;
+
+// LDS per wave: c [E] (the choice ranks; -inf once an expert is chosen or its group dropped) and
+// rank [n_groups] (-inf once a group is kept)
+__global__ void __launch_bounds__(256)
+route_groups_kernel(const float* __restrict__ z, const float* __restrict__ corr,
+                    float* __restrict__ out, int T, int E, int top, int n_groups, int keep,
+                    int rank_top, float scale, float sum_eps) {
+  extern __shared__ float s_all[];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int row = blockIdx.x * 4 + wv;
+  if (row >= T) return;                              // whole waves leave; no block barrier below
+  float* c = s_all + wv * (E + n_groups);
+  float* rank = c + E;
+  const float* zr = z + (long long)row * E;
+  float* orow = out + (long long)row * E;
+  for (int e = lane; e < E; e += 64) {
+    c[e] = sigmoid_f(zr[e]) + corr[e];
+    orow[e] = 0.f;
+  }
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  if (n_groups > 1 && keep < n_groups) {
+    const int per = E / n_groups;
+    // a group's rank: its `rank_top` largest c summed, one lane per group
+    for (int g = lane; g < n_groups; g += 64) {
+      float sum = 0.f;
+      int taken[4] = {-1, -1, -1, -1};               // rank_top <= 4
+      for (int r = 0; r < rank_top && r < per; ++r) {
+        float bv = -INFINITY;
+        int bi = -1;
+        for (int k = 0; k < per; ++k) {
+          bool used = false;
+          for (int q = 0; q < r; ++q) used |= taken[q] == k;
+          if (!used && (bi < 0 || c[g * per + k] > bv)) { bv = c[g * per + k]; bi = k; }
+        }
+        taken[r] = bi;
+        sum += bv;
+      }
+      rank[g] = sum;
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    for (int it = 0; it < keep; ++it) {
+      float bv = -INFINITY;
+      int bi = kNone;
+      for (int g = lane; g < n_groups; g += 64)
+        if (rank[g] > bv || (rank[g] == bv && g < bi && rank[g] != -INFINITY)) { bv = rank[g]; bi = g; }
+      wave_argmax(bv, bi);
+      if (bi == kNone) break;
+      if (lane == 0) rank[bi] = -INFINITY;           // kept: marked by -inf
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    }
+    for (int e = lane; e < E; e += 64)
+      if (rank[e / per] != -INFINITY) c[e] = -INFINITY;   // its group was not kept
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  }
+  float den = 0.f;
+  int mine[16];                                      // top <= E <= 1024: a lane wins <= 16 rounds
+  int n_mine = 0;
+  for (int it = 0; it < top; ++it) {
+    float bv = -INFINITY;
+    int bi = kNone;
+    for (int e = lane; e < E; e += 64)
+      if (c[e] > bv) { bv = c[e]; bi = e; }          // ascending e: ties keep the lowest index
+    wave_argmax(bv, bi);
+    if (bi == kNone) break;                          // fewer than `top` eligible experts
+    den += sigmoid_f(zr[bi]);
+    if ((bi & 63) == lane) {
+      c[bi] = -INFINITY;
+      if (n_mine < 16) mine[n_mine++] = bi;
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  }
+  const float k = scale / (den + sum_eps);
+  for (int q = 0; q < n_mine; ++q) orow[mine[q]] = sigmoid_f(zr[mine[q]]) * k;
+}
+
+template <typename T>
+__global__ void scaled_act_kernel(const T* __restrict__ u, const float* __restrict__ wts,
+                                  T* __restrict__ out, int Tn, int E, int ff, int ffs, int act) {
+  const int width = E * ff + ffs;
+  const long long n = (long long)Tn * width;
+  for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x) {
+    const int t = (int)(i / width), col = (int)(i % width);
+    const float w = col < E * ff ? wts[(long long)t * E + col / ff] : 1.f;
+    out[i] = from_f32<T>(w == 0.f ? 0.f : gate_act(to_f32(u[i]), act) * w);
+  }
+}
+
+// eight outputs per thread (16-byte accesses): block sizes multiples of 8, 16-bit dtypes
+template <typename T>
+__global__ void __launch_bounds__(256)
+scaled_act_v8(const T* __restrict__ u, const float* __restrict__ wts, T* __restrict__ out, int Tn,
+              int E, int ff, int ffs, int act) {
+  const int width = E * ff + ffs;
+  const int col = 8 * (blockIdx.x * 256 + threadIdx.x);
+  if (col >= width) return;
+  const int e = col < E * ff ? col / ff : -1;
+  for (int t = blockIdx.y; t < Tn; t += gridDim.y) {
+    const float w = e >= 0 ? wts[(long long)t * E + e] : 1.f;
+    float v[8], o[8];
+    if (w == 0.f) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = 0.f;
+    } else {
+      load8<T>(u + (long long)t * width + col, v);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = gate_act(v[j], act) * w;
+    }
+    store8<T>(out + (long long)t * width + col, o);
+  }
 }
 
 __global__ void __launch_bounds__(256)
@@ -148,6 +287,39 @@ hipError_t sm_route_topk(const float* z, float* out, int T, int E, int top, hipS
   if (T == 0) return hipSuccess;
   if (E < 1 || E > 64 * kMaxPerLane || top < 1 || top > E) return hipErrorInvalidValue;
   route_topk_kernel<<<(T + 3) / 4, 256, 0, st>>>(z, out, T, E, top);
+  return hipGetLastError();
+}
+
+// z, out [T, E] fp32; corr [E] fp32.  4 * (E + n_groups) * 4 bytes of LDS per workgroup.
+hipError_t sm_route_groups(const float* z, const float* corr, float* out, int T, int E, int top,
+                           int n_groups, int keep, int rank_top, float scale, float sum_eps,
+                           hipStream_t st) {
+  if (T == 0) return hipSuccess;
+  if (E < 1 || E > 64 * kMaxPerLane || n_groups < 1 || E % n_groups || keep < 1 ||
+      keep > n_groups || top < 1 || top > keep * (E / n_groups) || rank_top < 1 || rank_top > 4)
+    return hipErrorInvalidValue;
+  const size_t lds = 4 * (size_t)(E + n_groups) * sizeof(float);
+  route_groups_kernel<<<(T + 3) / 4, 256, lds, st>>>(z, corr, out, T, E, top, n_groups, keep,
+                                                     rank_top, scale, sum_eps);
+  return hipGetLastError();
+}
+
+hipError_t sm_scaled_act(int dt, const void* u, const float* wts, void* out, int T, int E, int ff,
+                         int ffs, int act, hipStream_t st) {
+  const long long n = (long long)T * (E * ff + ffs);
+  if (n == 0) return hipSuccess;
+  if (E > 0 && wts == nullptr) return hipErrorInvalidValue;
+  if (ff % 8 == 0 && ffs % 8 == 0 && (dt == kBF16 || dt == kF16)) {
+    const dim3 grid(((E * ff + ffs) / 8 + 255) / 256, T < 65535 ? T : 65535);
+    if (dt == kBF16)
+      scaled_act_v8<bf16><<<grid, 256, 0, st>>>((const bf16*)u, wts, (bf16*)out, T, E, ff, ffs, act);
+    else
+      scaled_act_v8<fp16><<<grid, 256, 0, st>>>((const fp16*)u, wts, (fp16*)out, T, E, ff, ffs, act);
+    return hipGetLastError();
+  }
+#define CALL(TT) scaled_act_kernel<TT><<<grid_for(n), 256, 0, st>>>((const TT*)u, wts, (TT*)out, T, E, ff, ffs, act)
+  SM_DISPATCH(dt, CALL)
+#undef CALL
   return hipGetLastError();
 }
 

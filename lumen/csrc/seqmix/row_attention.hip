@@ -7,14 +7,21 @@
 //                       part, rotated ] from the down projection's output into the paged cache
 //   sm_head_norm_write  q / k RMS norm per head with a weight shared by the heads: q in place,
 //                       normed k and plain v into their paged caches
+//   sm_row_norm_write   q / k RMS norm over the WHOLE projection (all heads at once) with weights
+//                       of that size: q in place, normed k into the key cache and k as projected
+//                       into the value cache (the values are the un-normalised keys)
 //   sm_row_attn         for every row t at position p and every query head h
 //        s_h(j)  = (q1_h . k_g(j)[0:D1] + q2_h . k_g(j)[D1:D1+D2]) * scale * temp(p)
 //        s_h(j) <- cap * tanh(s_h(j) / cap)                       (cap > 0)
 //        s_h(j) <- s_h(j) - r1_h * log(1 + r2_h * (p - j))        (r1 given)
+//        s_h(j) <- s_h(j) - slope_h * (p - j)                     (slopes given)
 //        s_h(j) <- sum_h' talk[h, h'] s_h'(j)                     (talk given)
-//        o_h     = sum_{j <= p} exp(s_h(j)) v_g(j) / (sum_{j <= p} exp(s_h(j)) + exp(sink_h))
+//        o_h     = sum_{j seen} exp(s_h(j)) v_g(j) / (sum_{j seen} exp(s_h(j)) + exp(sink_h))
+//        o_h    <- o_h * sigmoid(gate[t, h])                      (gate given)
 //     with temp(p) = 1 + tcoef * log(floor((p + 1) / tevery) + 1), g = h / (H / G), and the
-//     exp(sink_h) term only when a sink is given.  The query may come in two parts (two
+//     exp(sink_h) term only when a sink is given.  A row sees the keys j <= p; with a window > 0
+//     only those with p - j < window and, besides them, the first `keep` keys of the sequence: the
+//     64-key tiles that hold neither are skipped, so a row's cost is bounded by window + keep.  The query may come in two parts (two
 //     pointers with their own strides) that face the two parts of a key row; the value cache may
 //     be the key cache itself (a prefix of the key row is the value).  With G = 1 and D2 > 0 this
 //     is attention over a shared compressed key / value row (the query projected into the latent
@@ -185,6 +192,50 @@ head_norm_write_kernel(T* __restrict__ qkv, long long ld, const float* __restric
   }
 }
 
+// One workgroup per row: the sums of squares of the query part (HD entries) and of the key part
+// (GD entries) are reduced over the four waves in a fixed order, then q is normed in place and the
+// key goes to both caches.
+template <typename T>
+__global__ void __launch_bounds__(64 * kWaves)
+row_norm_write_kernel(T* __restrict__ qk, long long ld, const float* __restrict__ wq,
+                      const float* __restrict__ wk, const long long* __restrict__ slots,
+                      T* __restrict__ kcache, T* __restrict__ vcache, int HD, int GD, float eps) {
+  __shared__ float s_red[2][kWaves];
+  const int t = blockIdx.x, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const long long s = slots[t];
+  T* q = qk + (long long)t * ld;
+  const T* k = q + HD;
+  float sq = 0.f, sk = 0.f;
+  for (int c = threadIdx.x; c < HD; c += 64 * kWaves) {
+    const float v = to_f32(q[c]);
+    sq += v * v;
+  }
+  for (int c = threadIdx.x; c < GD; c += 64 * kWaves) {
+    const float v = to_f32(k[c]);
+    sk += v * v;
+  }
+  sq = wave_sum(sq);
+  sk = wave_sum(sk);
+  if (lane == 0) {
+    s_red[0][w] = sq;
+    s_red[1][w] = sk;
+  }
+  __syncthreads();
+  sq = (s_red[0][0] + s_red[0][1]) + (s_red[0][2] + s_red[0][3]);
+  sk = (s_red[1][0] + s_red[1][1]) + (s_red[1][2] + s_red[1][3]);
+  const float iq = 1.f / sqrtf(sq / (float)HD + eps), ik = 1.f / sqrtf(sk / (float)GD + eps);
+  if (s >= 0) {
+    T* kd = kcache + s * GD;
+    T* vd = vcache + s * GD;
+    for (int c = threadIdx.x; c < GD; c += 64 * kWaves) {
+      const T raw = k[c];
+      vd[c] = raw;
+      kd[c] = from_f32<T>(to_f32(raw) * ik * wk[c]);
+    }
+  }
+  for (int c = threadIdx.x; c < HD; c += 64 * kWaves) q[c] = from_f32<T>(to_f32(q[c]) * iq * wq[c]);
+}
+
 // Workgroups are handed to the 8 XCDs round-robin in launch order, and every XCD has an L2 of its
 // own.  Rows that follow each other in a step belong to one sequence and read the same cache
 // blocks, so XCD x takes the x-th CONTIGUOUS eighth of the rows instead of every eighth row:
@@ -206,8 +257,27 @@ struct RowAttnArgs {
   int H, G, HB, bs;
   float scale, softcap, tcoef; int tevery;
   const float *r1, *r2, *talk, *sink;
+  const float* slopes; int window, keep;     // linear distance bias; window + kept first keys
+  const T* gate; long long gater;            // per-head output gate logits [T][H], row stride
   int nsplit; float* ws_ml; float* ws_o;     // key splits: partial (max, sum) and accumulators
 };
+
+// The 64-key tiles a row at position `pos` visits: without a window all of 0 .. pos / 64; with one
+// the tiles of the first `keep` keys (as far as they lie below the window) and then those of the
+// window [pos - window + 1, pos].  Every visited tile holds at least one key the row sees.
+struct TileWalk {
+  int head, first, count;                    // tiles 0 .. head - 1, then first, first + 1, ...
+  __device__ __forceinline__ TileWalk(int pos, int window, int keep) {
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    first = lo / 64;
+    head = min((min(keep, lo) + 63) / 64, first);
+    count = head + pos / 64 - first + 1;
+  }
+  __device__ __forceinline__ int key0(int v) const { return 64 * (v < head ? v : first + v - head); }
+};
+__device__ __forceinline__ bool key_seen(int j, int pos, int window, int keep) {
+  return j <= pos && (window <= 0 || pos - j < window || j < keep);
+}
 
 // MMA (16-bit dtypes, key size and strides multiples of 8): the tile's scores come from the
 // matrix cores as S^T = K Q^T -- wave w takes keys 16 w .. 16 w + 15 of the tile against ALL
@@ -285,10 +355,12 @@ row_attn_kernel(const RowAttnArgs<T> a) {
   __syncthreads();
 
   int buf = 0;
-  for (int j0 = 64 * blockIdx.z; j0 <= pos; j0 += 64 * a.nsplit, buf ^= 1) {
+  const TileWalk walk(pos, a.window, a.keep);
+  for (int tv = blockIdx.z; tv < walk.count; tv += a.nsplit, buf ^= 1) {
+    const int j0 = walk.key0(tv);
     const int j = j0 + lane;
-    const bool valid = j <= pos;
-    const int rb = valid ? tbl[j / a.bs] * a.bs + j % a.bs : 0;
+    const bool valid = key_seen(j, pos, a.window, a.keep);
+    const int rb = j <= pos ? tbl[j / a.bs] * a.bs + j % a.bs : 0;
     if (w == 0) s_rb[buf * 64 + lane] = rb;
     const float dist = (float)(pos - j);
     if (MMA) {
@@ -319,7 +391,8 @@ row_attn_kernel(const RowAttnArgs<T> a) {
                 float sv = c[i] * qscale;
                 if (a.softcap > 0.f) sv = a.softcap * tanhf(sv / a.softcap);
                 if (a.r1 != nullptr) sv -= a.r1[h] * logf(1.f + a.r2[h] * (float)(pos - j0 - kk));
-                s_sc[(buf * a.HB + hl) * 64 + kk] = j0 + kk <= pos ? sv : 0.f;
+                if (a.slopes != nullptr) sv -= a.slopes[h] * (float)(pos - j0 - kk);
+                s_sc[(buf * a.HB + hl) * 64 + kk] = key_seen(j0 + kk, pos, a.window, a.keep) ? sv : 0.f;
               }
             }
           }
@@ -352,6 +425,7 @@ row_attn_kernel(const RowAttnArgs<T> a) {
         float sv = dot * qscale;
         if (a.softcap > 0.f) sv = a.softcap * tanhf(sv / a.softcap);
         if (a.r1 != nullptr) sv -= a.r1[h] * logf(1.f + a.r2[h] * dist);
+        if (a.slopes != nullptr) sv -= a.slopes[h] * dist;
         sv = valid ? sv : 0.f;
         sreg[i] = sv;
         s_sc[(buf * a.HB + hl) * 64 + lane] = sv;
@@ -370,7 +444,7 @@ row_attn_kernel(const RowAttnArgs<T> a) {
         for (int g = 0; g < nh; ++g) s += a.talk[h * a.H + h0 + g] * s_sc[(buf * a.HB + g) * 64 + lane];
       }
       s = valid ? s : -INFINITY;
-      const float mn = fmaxf(m[i], wave_max(s));          // finite: the tile's first key is valid
+      const float mn = fmaxf(m[i], wave_max(s));          // finite: a visited tile holds a seen key
       const float p = valid ? expf(s - mn) : 0.f;
       const float corr = expf(m[i] - mn);
       l[i] = l[i] * corr + wave_sum(p);
@@ -472,7 +546,8 @@ row_attn_kernel(const RowAttnArgs<T> a) {
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     }
     if (a.nsplit == 1) {
-      const float inv = 1.f / l[i];
+      float inv = 1.f / l[i];
+      if (a.gate != nullptr) inv *= sigmoid_f(to_f32(a.gate[(long long)t * a.gater + h]));
       T* op = a.out + (long long)t * a.our + (long long)h * a.ouh;
       for (int d = lane; d < a.Dv; d += 64) op[d] = from_f32<T>(so[d] * inv);
     } else {
@@ -698,12 +773,13 @@ hipError_t launch_latent_attn<float>(const RowAttnArgs<float>&, const float*, in
 }
 
 // out[t, h] = sum_s acc_s exp(m_s - M) / sum_s l_s exp(m_s - M), M = max_s m_s: the splits of a
-// row's keys merged; a split that saw no key has (m, l) = (-inf, 0) and drops out
+// row's keys merged; a split that saw no key has (m, l) = (-inf, 0) and drops out.  With a gate
+// the head's output is multiplied by sigmoid(gate[t, h]).
 template <typename T>
 __global__ void __launch_bounds__(256)
 row_attn_combine_kernel(const float* __restrict__ ws_ml, const float* __restrict__ ws_o,
                         T* __restrict__ out, long long our, long long ouh, int H, int Dv,
-                        int nsplit) {
+                        int nsplit, const T* __restrict__ gate, long long gater) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63;
   const long long base = ((long long)t * H + h) * nsplit;
   __shared__ float s_w[64];
@@ -712,7 +788,8 @@ row_attn_combine_kernel(const float* __restrict__ ws_ml, const float* __restrict
     const float ls = lane < nsplit ? ws_ml[2 * (base + lane) + 1] : 0.f;
     const float M = wave_max(ms);
     const float e = ms == -INFINITY ? 0.f : expf(ms - M);
-    const float L = wave_sum(ls * e);
+    float L = wave_sum(ls * e);
+    if (gate != nullptr) L *= 1.f + expf(-to_f32(gate[(long long)t * gater + h]));   // / sigmoid
     s_w[lane] = e / L;
   }
   __syncthreads();
@@ -765,7 +842,7 @@ hipError_t launch_row_attn(const RowAttnArgs<T>& a, int Tn, hipStream_t st) {
 #undef LAUNCH
   if (a.nsplit > 1)
     row_attn_combine_kernel<T><<<dim3(Tn, a.H), 256, 0, st>>>(a.ws_ml, a.ws_o, a.out, a.our, a.ouh,
-                                                              a.H, a.Dv, a.nsplit);
+                                                              a.H, a.Dv, a.nsplit, a.gate, a.gater);
   return hipGetLastError();
 }
 
@@ -819,6 +896,19 @@ hipError_t sm_head_norm_write(int dt, void* qkv, long long ld, const float* wq, 
   return hipGetLastError();
 }
 
+// qk [T, >= HD + GD] (row stride ld): q normed in place over its HD entries with wq [HD]; the key
+// part normed with wk [GD] into kcache and copied as projected into vcache, both [rows, GD].
+hipError_t sm_row_norm_write(int dt, void* qk, long long ld, const float* wq, const float* wk,
+                             const long long* slots, void* kcache, void* vcache, int T, int HD,
+                             int GD, float eps, hipStream_t st) {
+  if (T == 0) return hipSuccess;
+  if (HD < 1 || GD < 1 || ld < HD + GD) return hipErrorInvalidValue;
+#define CALL(TT) row_norm_write_kernel<TT><<<T, 64 * kWaves, 0, st>>>((TT*)qk, ld, wq, wk, slots, (TT*)kcache, (TT*)vcache, HD, GD, eps)
+  SM_DISPATCH(dt, CALL)
+#undef CALL
+  return hipGetLastError();
+}
+
 // 1 when sm_latent_attn has a kernel for these sizes (dtype code dt, value size Dv = the latent,
 // key size Dk, cache block bs), else 0: the caller then takes sm_row_attn
 int sm_latent_attn_ok(int dt, int Dv, int Dk, int D1, int bs) {
@@ -852,12 +942,13 @@ hipError_t sm_latent_attn(int dt, const void* q1, long long q1r, long long q1h, 
     RowAttnArgs<TT> a{(const TT*)q1, q1r, q1h, D1, (const TT*)q2, q2r, q2h, D2,               \
                       (const TT*)kc, krow, (const TT*)kc, krow, Dv, (TT*)out, our, ouh,       \
                       tables, maxb, row_seg, positions, H, 1, 16, bs, scale, softcap, tcoef,  \
-                      tevery, r1, r2, nullptr, sink, nsplit, ws_ml, ws_o};                    \
+                      tevery, r1, r2, nullptr, sink, nullptr, 0, 0, nullptr, 0, nsplit,       \
+                      ws_ml, ws_o};                                                           \
     hipError_t e = launch_latent_attn<TT>(a, (const TT*)vt, T, st);                           \
     if (e != hipSuccess) return e;                                                            \
     if (nsplit > 1)                                                                           \
-      row_attn_combine_kernel<TT><<<dim3(T, H), 256, 0, st>>>(ws_ml, ws_o, (TT*)out, our,     \
-                                                              ouh, H, Dv, nsplit);            \
+      row_attn_combine_kernel<TT><<<dim3(T, H), 256, 0, st>>>(                                \
+          ws_ml, ws_o, (TT*)out, our, ouh, H, Dv, nsplit, (const TT*)nullptr, 0ll);           \
     return hipGetLastError();                                                                 \
   }
   SM_DISPATCH(dt, CALL)
@@ -875,18 +966,20 @@ hipError_t sm_row_attn(int dt, const void* q1, long long q1r, long long q1h, int
                        const int* row_seg, const int* positions, int T, int H, int G, int HB,
                        int bs, float scale, float softcap, float tcoef, int tevery,
                        const float* r1, const float* r2, const float* talk, const float* sink,
-                       int nsplit, float* ws_ml, float* ws_o, hipStream_t st) {
+                       const float* slopes, int window, int keep, const void* gate,
+                       long long gater, int nsplit, float* ws_ml, float* ws_o, hipStream_t st) {
   if (T == 0) return hipSuccess;
   if (nsplit < 1 || nsplit > 64 || (nsplit > 1 && (!ws_ml || !ws_o))) return hipErrorInvalidValue;
   if (H % G != 0 || HB < 1 || HB > 8 * kWaves || Dv > kMaxDv || (talk && HB < H) ||
-      (D2 > 0 && q2 == nullptr))
+      (D2 > 0 && q2 == nullptr) || window < 0 || keep < 0)
     return hipErrorInvalidValue;
 #define CALL(TT)                                                                              \
   {                                                                                           \
     RowAttnArgs<TT> a{(const TT*)q1, q1r, q1h, D1, (const TT*)q2, q2r, q2h, D2,               \
                       (const TT*)kc, krow, (const TT*)vc, vrow, Dv, (TT*)out, our, ouh,       \
                       tables, maxb, row_seg, positions, H, G, HB, bs, scale, softcap, tcoef,  \
-                      tevery, r1, r2, talk, sink, nsplit, ws_ml, ws_o};                                         \
+                      tevery, r1, r2, talk, sink, slopes, window, keep, (const TT*)gate,      \
+                      gater, nsplit, ws_ml, ws_o};                                            \
     return launch_row_attn<TT>(a, T, st);                                                     \
   }
   SM_DISPATCH(dt, CALL)

@@ -17,7 +17,7 @@ from typing import Optional
 
 @dataclass
 class ModelConfig:
-    arch: str = "llama"  # "llama" | "opt" | "gedatar" | "dalavik"
+    arch: str = "llama"  # "llama" | "opt" | "gedatar" | "dalavik" | "fanopel"
     vocab_size: int = 32000
     hidden_size: int = 4096
     intermediate_size: int = 11008
@@ -46,12 +46,16 @@ class ModelConfig:
     # and the per-layer width of the second, per-token embedding (0: the design's side input is off)
     norm_groups: int = 1
     token_side_dim: int = 0
+    # Fanopel (layer_specs of gated window attention + routed experts; learned positions, so
+    # max_position_embeddings is the position table's row count): every sublayer's output is
+    # multiplied by this before it joins the residual stream
+    residual_mult: float = 1.0
 
     @property
     def is_hybrid(self) -> bool:
         """Every layer names its own mixer and keeps its own kind of cache or state; such a stack
         is served by ``serve.hybrid_runner`` on the step's row segments."""
-        return self.arch in ("gedatar", "dalavik")
+        return self.arch in ("gedatar", "dalavik", "fanopel")
 
     @property
     def head_dim(self) -> int:
@@ -71,6 +75,8 @@ class ModelConfig:
         if self.is_hybrid:
             if self.arch == "gedatar":
                 from .gedatar import tensor_shapes
+            elif self.arch == "fanopel":
+                from .fanopel import tensor_shapes
             else:
                 from .dalavik import tensor_shapes
 
@@ -165,7 +171,39 @@ def dalavik_to_dict(cfg: ModelConfig) -> dict:
     return d
 
 
+def _fanopel_to_config(d: dict) -> ModelConfig:
+    """config.json of a Fanopel checkpoint: {"architecture": "Fanopel", "vocab", "width",
+    "max_positions", "residual_mult", "norm": {"eps"}, "layers": [{"type", "mixer", "mlp"}, ...]}."""
+    layers = d["layers"]
+    if not layers:
+        raise ValueError("a Fanopel config needs at least one layer")
+    for i, L in enumerate(layers):
+        if L.get("type") != "attention":
+            raise ValueError(f"layer {i}: unknown mixer type {L.get('type')!r}")
+        kind = (L.get("mlp") or {}).get("kind", None)
+        if L.get("mlp") is not None and kind != "moe":
+            raise ValueError(f"layer {i}: unknown feed-forward kind {kind!r}")
+    return ModelConfig(
+        arch="fanopel", vocab_size=int(d["vocab"]), hidden_size=int(d["width"]),
+        num_hidden_layers=len(layers), rms_norm_eps=float(d["norm"]["eps"]),
+        residual_mult=float(d.get("residual_mult", 1.0)), layer_specs=layers,
+        intermediate_size=0, num_attention_heads=0, num_key_value_heads=0,
+        max_position_embeddings=int(d["max_positions"]),
+        bos_token_id=int(d.get("bos_token_id", 0)), eos_token_id=int(d.get("eos_token_id", -1)),
+        pad_token_id=int(d.get("pad_token_id", 0)), name=d.get("_name_or_path", "fanopel"))
+
+
+def fanopel_to_dict(cfg: ModelConfig) -> dict:
+    """The checkpoint form of a Fanopel configuration (inverse of ``_fanopel_to_config``)."""
+    return {"architecture": "Fanopel", "vocab": cfg.vocab_size, "width": cfg.hidden_size,
+            "max_positions": cfg.max_position_embeddings, "residual_mult": cfg.residual_mult,
+            "norm": {"eps": cfg.rms_norm_eps}, "layers": cfg.layer_specs,
+            "eos_token_id": cfg.eos_token_id}
+
+
 def _hf_to_config(d: dict) -> ModelConfig:
+    if d.get("architecture") == "Fanopel":
+        return _fanopel_to_config(d)
     if d.get("architecture") == "Gedatar":
         return _gedatar_to_config(d)
     if d.get("architecture") == "Dalavik":
@@ -285,6 +323,29 @@ PRESETS = {
                                             "scale": 0.18, "softcap": 30.0,
                                             "q_temp": {"coef": 0.1, "every": 7}},
              "mlp": {"kind": "dense", "ff": 96}}]),
+    # gated window attention (whole-projection q / k norms, keys as values, soft cap, linear
+    # distance bias, kept first tokens) + sigmoid-routed experts chosen within the best groups;
+    # learned positions; one layer without a feed-forward
+    "tiny-fanopel": dict(
+        arch="fanopel", vocab_size=272, hidden_size=112, num_hidden_layers=3, rms_norm_eps=1e-5,
+        residual_mult=0.7, intermediate_size=0, num_attention_heads=0, num_key_value_heads=0,
+        max_position_embeddings=384, eos_token_id=-1, name="tiny-fanopel", layer_specs=[
+            {"type": "attention", "mixer": {"heads": 6, "kv_heads": 3, "dim": 24, "vdim": 24,
+                                            "scale": 0.2, "softcap": 20.0,
+                                            "mask": {"size": 21, "keep_first": 3}},
+             "mlp": {"kind": "moe", "expert": {"ff": 40},
+                     "router": {"experts": 12, "top": 4, "scale": 1.5,
+                                "groups": {"count": 4, "keep": 2}}}},
+            {"type": "attention", "mixer": {"heads": 2, "kv_heads": 1, "dim": 32, "vdim": 32,
+                                            "scale": 0.18, "softcap": 8.0,
+                                            "mask": {"size": 70, "keep_first": 1}},
+             "mlp": None},
+            {"type": "attention", "mixer": {"heads": 4, "kv_heads": 4, "dim": 16, "vdim": 16,
+                                            "scale": 0.25, "softcap": 50.0,
+                                            "mask": {"size": 9, "keep_first": 5}},
+             "mlp": {"kind": "moe", "expert": {"ff": 56},
+                     "router": {"experts": 5, "top": 2, "scale": 1.0,
+                                "groups": {"count": 1, "keep": 1}}}}]),
     "tiny-opt": dict(arch="opt", vocab_size=512, hidden_size=64, intermediate_size=256,
                      ffn_dim=256, num_hidden_layers=2, num_attention_heads=4,
                      num_key_value_heads=4, max_position_embeddings=256, word_embed_proj_dim=64,

@@ -79,6 +79,10 @@ def load_hf_weights(model: nn.Module, path: str, strict: bool = True) -> None:
         from .dalavik import load_dalavik_weights
 
         return load_dalavik_weights(model, handles, path)
+    if model.config.arch == "fanopel":
+        from .fanopel import load_fanopel_weights
+
+        return load_fanopel_weights(model, handles, path)
     params = dict(model.named_parameters())
     for ours, srcs in _hf_name_map(model).items():
         if ours not in params:
@@ -108,13 +112,14 @@ def save_hf_weights(model: nn.Module, path: str, shard_bytes: int = 5 << 30) -> 
     os.makedirs(path, exist_ok=True)
     cfg = model.config
     if cfg.is_hybrid:
-        from .config import dalavik_to_dict, gedatar_to_dict
+        from .config import dalavik_to_dict, fanopel_to_dict, gedatar_to_dict
 
         save_file({n: model.tensor(n).detach().cpu().contiguous() for n in model.tensor_names()},
                   os.path.join(path, "model.safetensors"), metadata={"format": "pt"})
         with open(os.path.join(path, "config.json"), "w") as f:
-            json.dump((gedatar_to_dict if cfg.arch == "gedatar" else dalavik_to_dict)(cfg), f,
-                      indent=2)
+            to_dict = {"gedatar": gedatar_to_dict, "dalavik": dalavik_to_dict,
+                       "fanopel": fanopel_to_dict}[cfg.arch]
+            json.dump(to_dict(cfg), f, indent=2)
         return
     params = dict(model.named_parameters())
     out: Dict[str, torch.Tensor] = {}

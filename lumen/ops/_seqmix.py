@@ -39,7 +39,13 @@ SIGNATURES = {
     "sm_latent_write": "iplppppppiiiiif",
     "sm_head_norm_write": "iplpppppiiiiif",
     "sm_latent_attn": "i" "plli" "plli" "pl" "pi" "pll" "pi" "pp" "iii" "fffi" "ppp" "ipp",
-    "sm_row_attn": "i" "plli" "plli" "pl" "pli" "pll" "pi" "pp" "iiiii" "fffi" "pppp" "ipp",
+    "sm_row_attn": "i" "plli" "plli" "pl" "pli" "pll" "pi" "pp" "iiiii" "fffi" "pppp" "piipl"
+                   "ipp",
+    "sm_row_norm_write": "iplpppppiiif",
+    "sm_layer_norm": "iippfppiif",
+    "sm_embed_pos": "ipppppiiii",
+    "sm_route_groups": "pppiiiiiiff",
+    "sm_scaled_act": "ipppiiiii",
 }
 
 

@@ -674,8 +674,47 @@ def head_norm_write(qkv: torch.Tensor, wq: torch.Tensor, wk: torch.Tensor, slots
          qkv.shape[0], H, G, D, Dv, eps)
 
 
+def row_norm_write_ref(qk, wq, wk, slots, kcache, vcache, HD, GD, eps):
+    def unit(x):
+        x = x.float()
+        return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+
+    k = qk[:, HD:HD + GD]
+    ok = slots >= 0
+    vcache.view(-1, GD)[slots[ok]] = k[ok].to(vcache.dtype)
+    kcache.view(-1, GD)[slots[ok]] = (unit(k) * wk.float())[ok].to(kcache.dtype)
+    qk[:, :HD] = (unit(qk[:, :HD]) * wq.float()).to(qk.dtype)
+
+
+def row_norm_write(qk: torch.Tensor, wq: torch.Tensor, wk: torch.Tensor, slots: torch.Tensor,
+                   kcache: torch.Tensor, vcache: torch.Tensor, HD: int, GD: int,
+                   eps: float) -> None:
+    """qk [T, >= HD + GD] (a fused projection's output; further columns are left alone): the
+    query part [0, HD) is RMS-normed over ALL its HD entries at once (every head together) with
+    the weight ``wq`` [HD] and replaced in place; the key part [HD, HD + GD) goes to the paged
+    caches at ``slots`` (int64; -1 skips) twice: normed the same way with ``wk`` [GD] into
+    ``kcache``, and as projected into ``vcache`` (the values are the un-normalised keys).  Both
+    caches are [blocks, block, G, D] with G * D = GD."""
+    from ._seqmix import DT, call, use_seqmix
+
+    if qk.shape[1] < HD + GD:
+        raise ValueError(f"qk has {qk.shape[1]} columns, expected at least {HD + GD}")
+    if kcache.shape[2:].numel() != GD or vcache.shape[2:].numel() != GD:
+        raise ValueError(f"cache rows of {kcache.shape[2:].numel()} / {vcache.shape[2:].numel()} "
+                         f"do not hold keys of {GD}")
+    if not use_seqmix(qk):
+        return row_norm_write_ref(qk, wq, wk, slots, kcache, vcache, HD, GD, eps)
+    assert qk.stride(1) == 1 and kcache.is_contiguous() and vcache.is_contiguous()
+    assert kcache.dtype == qk.dtype and vcache.dtype == qk.dtype
+    assert wq.dtype == torch.float32 and wk.dtype == torch.float32
+    assert tuple(wq.shape) == (HD,) and tuple(wk.shape) == (GD,)
+    call("sm_row_norm_write", DT[qk.dtype], qk, qk.stride(0), wq, wk, slots, kcache, vcache,
+         qk.shape[0], HD, GD, eps)
+
+
 def row_attention_ref(q1, q2, kcache, vcache, Dv, out, seg, H, G, scale, softcap=0.0,
-                      q_temp=None, r1=None, r2=None, talk=None, sink=None):
+                      q_temp=None, r1=None, r2=None, talk=None, sink=None, slopes=None,
+                      window=0, keep_first=0, gate=None):
     T = q1.shape[0]
     D1 = q1.shape[2]
     D2 = q2.shape[2] if q2 is not None else 0
@@ -689,6 +728,8 @@ def row_attention_ref(q1, q2, kcache, vcache, Dv, out, seg, H, G, scale, softcap
     for t in range(T):
         p = pos[t]
         js = torch.arange(0, p + 1, device=q.device)
+        if window and window > 0:
+            js = js[(p - js < window) | (js < keep_first)]
         tbl = seg.tables[row_seg[t]].long()
         rows = tbl[js // bs] * bs + js % bs
         k = krows[rows][:, :G * Dk].float().view(-1, G, Dk)[:, hg]              # [n, H, Dk]
@@ -704,6 +745,8 @@ def row_attention_ref(q1, q2, kcache, vcache, Dv, out, seg, H, G, scale, softcap
         if r1 is not None:
             d = (p - js).float()
             s = s - r1.float().view(H, 1) * torch.log(1.0 + r2.float().view(H, 1) * d)
+        if slopes is not None:
+            s = s - slopes.float().view(H, 1) * (p - js).float()
         if talk is not None:
             s = talk.float() @ s
         m = s.max(-1, keepdim=True).values
@@ -713,7 +756,10 @@ def row_attention_ref(q1, q2, kcache, vcache, Dv, out, seg, H, G, scale, softcap
         den = e.sum(-1, keepdim=True)
         if sink is not None:
             den = den + torch.exp(sink.float().view(H, 1) - m)
-        out[t] = torch.einsum("hn,nhd->hd", e / den, v).to(out.dtype)
+        o = torch.einsum("hn,nhd->hd", e / den, v)
+        if gate is not None:
+            o = o * torch.sigmoid(gate[t].float()).view(H, 1)
+        out[t] = o.to(out.dtype)
     return out
 
 
@@ -736,7 +782,8 @@ def _heads_per_block(H: int, Dk: int, need_all: bool) -> int:
 def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Tensor,
                   vcache: torch.Tensor, Dv: int, out: torch.Tensor, seg, H: int, G: int,
                   scale: float, softcap: float = 0.0, q_temp=None, r1=None, r2=None, talk=None,
-                  sink=None, vt: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  sink=None, vt: Optional[torch.Tensor] = None, slopes=None, window: int = 0,
+                  keep_first: int = 0, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention of every row of a step against paged caches.
 
     q1 [T, H, D1] and (optionally) q2 [T, H, D2] are views with arbitrary row / head strides;
@@ -748,7 +795,11 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
     multiplied by 1 + coef * ln(floor((p + 1) / every) + 1).  ``softcap`` > 0: s <- cap *
     tanh(s / cap).  ``r1``, ``r2`` [H]: s <- s - r1 * ln(1 + r2 * distance).  ``talk`` [H, H]:
     the heads' scores are mixed, s_h <- sum_g talk[h, g] s_g.  ``sink`` [H]: exp(sink_h) joins
-    the softmax denominator.  ``vt`` [blocks, Dv, block]: a per-block transposed copy of the
+    the softmax denominator.  ``slopes`` [H]: s <- s - slopes_h * distance (a linear distance
+    bias).  ``window`` > 0: a row at position p only sees the keys j with p - j < window and,
+    besides them, the sequence's first ``keep_first`` keys (at their true distances); tiles of
+    keys between the two ranges are never loaded.  ``gate`` [T, H] (a view, any row stride):
+    head h's output is multiplied by sigmoid(gate[t, h]).  ``vt`` [blocks, Dv, block]: a per-block transposed copy of the
     values (``latent_write`` keeps one); with it, one key/value head, values that are a prefix of
     the key rows and a 16-bit dtype, the whole kernel runs on the matrix cores."""
     from ._seqmix import DT, call, latent_attn_ok, use_seqmix
@@ -760,7 +811,7 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
         raise ValueError(f"{H} heads are not a multiple of {G} key/value heads")
     if not use_seqmix(q1):
         return row_attention_ref(q1, q2, kcache, vcache, Dv, out, seg, H, G, scale, softcap,
-                                 q_temp, r1, r2, talk, sink)
+                                 q_temp, r1, r2, talk, sink, slopes, window, keep_first, gate)
     if Dv > 512:
         raise ValueError(f"value size {Dv} > 512 is not supported")
     assert kcache.is_contiguous() and vcache.is_contiguous() and kcache.dtype == q1.dtype
@@ -768,12 +819,16 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
     krow = kcache.shape[2:].numel()
     vrow = vcache.shape[2:].numel()
     assert krow >= G * Dk and vrow >= G * Dv
-    for f in (r1, r2, talk, sink):
+    for f in (r1, r2, talk, sink, slopes):
         assert f is None or (f.dtype == torch.float32 and f.is_contiguous())
+    window, keep_first = max(0, int(window or 0)), max(0, int(keep_first or 0))
+    if gate is not None:
+        assert gate.dtype == q1.dtype and gate.stride(1) == 1 and tuple(gate.shape) == (T, H)
     coef, every = (float(q_temp[0]), int(q_temp[1])) if q_temp is not None else (0.0, 0)
     bs = kcache.shape[1]
     al8 = lambda x: x.data_ptr() % 16 == 0 and x.stride(0) % 8 == 0 and x.stride(1) % 8 == 0  # noqa: E731
     if (vt is not None and G == 1 and talk is None and vcache is kcache and D1 >= Dv
+            and slopes is None and window == 0 and gate is None
             and q1.dtype in (torch.bfloat16, torch.float16) and latent_attn_ok(DT[q1.dtype], Dv, Dk, D1, bs)
             and krow % 8 == 0 and al8(q1) and (q2 is None or al8(q2)) and out.data_ptr() % 8 == 0
             and out.stride(0) % 4 == 0 and out.stride(1) % 4 == 0):
@@ -795,6 +850,8 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
     # few rows (decoding): deal a row's 64-key tiles out to several workgroups so that ~2 per CU
     # run; the count depends on the step's size only, never on device data (graph capture)
     tiles = (seg.tables.shape[1] * kcache.shape[1] + 63) // 64
+    if window > 0:                     # a row visits the window's tiles and the kept first ones
+        tiles = min(tiles, (window + 63) // 64 + 1 + (keep_first + 63) // 64)
     while talk is None and HB > 4 and T * ((H + HB - 1) // HB) * tiles < 512:
         HB //= 2                       # fewer heads per workgroup: more workgroups
     blocks = T * ((H + HB - 1) // HB)
@@ -808,5 +865,6 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
          kcache, krow, vcache, vrow, Dv, out, out.stride(0), out.stride(1),
          seg.tables, seg.tables.shape[1], seg.row_seg, seg.positions, T, H, G, HB,
          kcache.shape[1], scale, float(softcap or 0.0), coef, every, r1, r2, talk, sink,
+         slopes, window, keep_first, gate, gate.stride(0) if gate is not None else 0,
          nsplit, ws_ml, ws_o)
     return out

@@ -46,3 +46,26 @@ def gated_token_slice(z: torch.Tensor, table: torch.Tensor, tokens: torch.Tensor
     call("sm_gate_rows", DT[z.dtype], z, z.stride(0), table, table.stride(0), tokens, col0, dim,
          out, T)
     return out
+
+
+def embed_positions_ref(tokens, positions, table, pos_table):
+    return table[tokens].float() + pos_table[positions.long()].float()
+
+
+def embed_positions(tokens: torch.Tensor, positions: torch.Tensor, table: torch.Tensor,
+                    pos_table: torch.Tensor) -> torch.Tensor:
+    """table[token] + pos_table[position] per row, summed in fp32: the start of a residual stream
+    with learned positions, [T, W] fp32.  ``positions`` must be below the position table's row
+    count (the caller's length limit guarantees it).  (HIP ``csrc/seqmix/layer_norm.hip``.)"""
+    from ._seqmix import DT, call, use_seqmix
+
+    if not use_seqmix(table):
+        return embed_positions_ref(tokens, positions, table, pos_table)
+    assert table.is_contiguous() and pos_table.is_contiguous() and table.dtype == pos_table.dtype
+    assert tokens.dtype == torch.int64 and tokens.is_contiguous()
+    assert positions.dtype == torch.int32 and positions.is_contiguous()
+    T, W = tokens.shape[0], table.shape[1]
+    out = torch.empty(T, W, dtype=torch.float32, device=table.device)
+    call("sm_embed_pos", DT[table.dtype], table, pos_table, tokens, positions, out, T, W,
+         table.shape[0], pos_table.shape[0])
+    return out

@@ -45,8 +45,53 @@ def route_topk(z: torch.Tensor, top: int) -> torch.Tensor:
     return out
 
 
-GATE_ACTS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
-_ACT_FN = {"silu": F.silu, "relu": F.relu, "gelu_tanh": lambda z: F.gelu(z, approximate="tanh")}
+def route_groups_ref(z, correction, top, n_groups, keep, scale, sum_eps=1e-20, rank_top=2):
+    T, E = z.shape
+    s = torch.sigmoid(z.float())
+    c = s + correction.float()
+    if n_groups > 1 and keep < n_groups:
+        per = E // n_groups
+        cg = c.view(T, n_groups, per)
+        rank = torch.sort(cg, dim=-1, descending=True).values[..., :min(rank_top, per)].sum(-1)
+        best = torch.sort(rank, dim=-1, descending=True, stable=True).indices[:, :keep]
+        allow = torch.zeros(T, n_groups, dtype=torch.bool, device=z.device).scatter_(1, best, True)
+        c = cg.masked_fill(~allow.view(T, n_groups, 1), float("-inf")).reshape(T, E)
+    idx = torch.sort(c, dim=-1, descending=True, stable=True).indices[:, :top]
+    chosen = torch.gather(s, 1, idx)
+    wt = chosen / (chosen.sum(-1, keepdim=True) + sum_eps) * scale
+    return torch.zeros_like(s).scatter_(1, idx, wt)
+
+
+def route_groups(z: torch.Tensor, correction: torch.Tensor, top: int, n_groups: int, keep: int,
+                 scale: float, sum_eps: float = 1e-20, rank_top: int = 2) -> torch.Tensor:
+    """Router logits z [T, E] (fp32) -> dense routing weights [T, E] (fp32) of a sigmoid router
+    with a choice correction and a limit to the best groups: the scores are s = sigmoid(z); the
+    choice ranks c = s + ``correction`` [E]; the experts form ``n_groups`` equal groups of
+    neighbours, a group ranks by the sum of its ``rank_top`` largest c, and only experts of the
+    ``keep`` best groups can be chosen (``keep`` = ``n_groups``: no limit); the ``top`` eligible
+    experts with the largest c get s_e / (sum of the chosen s + ``sum_eps``) * ``scale`` at their
+    places, all others zero.  Ties go to the lowest index."""
+    from ._seqmix import call, use_seqmix
+
+    T, E = z.shape
+    if n_groups < 1 or E % n_groups or not 1 <= keep <= n_groups:
+        raise ValueError(f"{E} experts do not form {n_groups} equal groups of which {keep} are kept")
+    if not 1 <= top <= keep * (E // n_groups):
+        raise ValueError(f"top {top} exceeds the {keep * (E // n_groups)} eligible experts")
+    if not use_seqmix(z):
+        return route_groups_ref(z, correction, top, n_groups, keep, scale, sum_eps, rank_top)
+    assert z.dtype == torch.float32 and z.is_contiguous()
+    assert correction.dtype == torch.float32 and correction.is_contiguous()
+    if E > 1024:
+        raise ValueError(f"route_groups supports at most 1024 experts, got {E}")
+    out = torch.empty_like(z)
+    call("sm_route_groups", z, correction, out, T, E, top, n_groups, keep, rank_top, scale, sum_eps)
+    return out
+
+
+GATE_ACTS = {"silu": 0, "relu": 1, "gelu_tanh": 2, "relu2": 3}
+_ACT_FN = {"silu": F.silu, "relu": F.relu, "gelu_tanh": lambda z: F.gelu(z, approximate="tanh"),
+           "relu2": lambda z: F.relu(z) ** 2}
 
 
 def gated_act_ref(gu, wts, E, ff, ffs, act="silu"):
@@ -78,13 +123,48 @@ def gated_act(gu: torch.Tensor, wts: Optional[torch.Tensor], E: int, ff: int,
     return out
 
 
-def moe_dense(h, wts, gu_w, down_w, E: int, ff: int, ffs: int) -> torch.Tensor:
-    return F.linear(gated_act(F.linear(h, gu_w), wts, E, ff, ffs), down_w)
+def scaled_act_ref(u, wts, E, ff, ffs, act="relu2"):
+    T = u.shape[0]
+    fn = _ACT_FN[act]
+    parts = []
+    if E:
+        parts.append((fn(u[:, :E * ff].float()).view(T, E, ff) * wts.float()[:, :, None])
+                     .reshape(T, E * ff))
+    if ffs:
+        parts.append(fn(u[:, E * ff:].float()))
+    return torch.cat(parts, 1).to(u.dtype)
 
 
-def moe_grouped(h, wts, gu_w, down_w, E: int, ff: int, ffs: int) -> torch.Tensor:
+def scaled_act(u: torch.Tensor, wts: Optional[torch.Tensor], E: int, ff: int, ffs: int,
+               act: str = "relu2") -> torch.Tensor:
+    """act(u) over the stacked up projections of experts WITHOUT a gate (``act``: as for
+    ``gated_act``, plus relu2 = relu(.)^2): ``u`` [T, E * ff + ffs] holds E expert blocks of ff and
+    one unweighted block of ffs; expert e's activation is scaled by ``wts[:, e]``.  Same shape
+    out."""
+    from ._seqmix import DT, call, use_seqmix
+
+    if not use_seqmix(u):
+        return scaled_act_ref(u, wts, E, ff, ffs, act)
+    assert u.is_contiguous() and u.shape[1] == E * ff + ffs
+    out = torch.empty_like(u)
+    call("sm_scaled_act", DT[u.dtype], u, wts, out, u.shape[0], E, ff, ffs, GATE_ACTS[act])
+    return out
+
+
+def _act(z, wts, E, ff, ffs, act, gated):
+    return (gated_act if gated else scaled_act)(z, wts, E, ff, ffs, act)
+
+
+def moe_dense(h, wts, gu_w, down_w, E: int, ff: int, ffs: int, act: str = "silu",
+              gated: bool = True) -> torch.Tensor:
+    return F.linear(_act(F.linear(h, gu_w), wts, E, ff, ffs, act, gated), down_w)
+
+
+def moe_grouped(h, wts, gu_w, down_w, E: int, ff: int, ffs: int, act: str = "silu",
+                gated: bool = True) -> torch.Tensor:
     """Same result as ``moe_dense`` (to rounding) running each expert on its own rows only."""
     T = h.shape[0]
+    k = 2 if gated else 1                                 # rows of the first weight per ff
     tok, exp = (wts > 0).nonzero(as_tuple=True)           # (host sync) pairs in token order
     order = torch.argsort(exp, stable=True)
     tok, exp = tok[order], exp[order]
@@ -96,14 +176,14 @@ def moe_grouped(h, wts, gu_w, down_w, E: int, ff: int, ffs: int) -> torch.Tensor
     a = 0
     for e, n in enumerate(counts):
         if n:
-            gu = F.linear(x[a:a + n], gu_w[e * 2 * ff:(e + 1) * 2 * ff])
-            torch.matmul(gated_act(gu, None, 0, 0, ff), down_w[:, e * ff:(e + 1) * ff].t(),
+            gu = F.linear(x[a:a + n], gu_w[e * k * ff:(e + 1) * k * ff])
+            torch.matmul(_act(gu, None, 0, 0, ff, act, gated), down_w[:, e * ff:(e + 1) * ff].t(),
                          out=ys[a:a + n])
             a += n
     out.index_add_(0, tok, ys.float() * wsel)
     if ffs:
-        gu = F.linear(h, gu_w[E * 2 * ff:])
-        out += F.linear(gated_act(gu, None, 0, 0, ffs), down_w[:, E * ff:]).float()
+        gu = F.linear(h, gu_w[E * k * ff:])
+        out += F.linear(_act(gu, None, 0, 0, ffs, act, gated), down_w[:, E * ff:]).float()
     return out.to(h.dtype)
 
 
@@ -111,8 +191,11 @@ def moe_grouped(h, wts, gu_w, down_w, E: int, ff: int, ffs: int) -> torch.Tensor
 GROUPED_MIN_ROWS = 256
 
 
-def moe(h, wts, gu_w, down_w, E: int, top: int, ff: int, ffs: int) -> torch.Tensor:
-    """Weighted sum of each row's chosen experts (+ the shared expert): [T, W] in h's dtype."""
+def moe(h, wts, gu_w, down_w, E: int, top: int, ff: int, ffs: int, act: str = "silu",
+        gated: bool = True) -> torch.Tensor:
+    """Weighted sum of each row's chosen experts (+ the shared expert): [T, W] in h's dtype.
+    ``gated``: an expert is W_down (act(W_gate h) * W_up h) with [gate | up] rows stacked per
+    expert in ``gu_w``; else W_down act(W_up h) with the up rows alone."""
     grouped = (h.shape[0] >= GROUPED_MIN_ROWS and top * 2 <= E
                and not (h.is_cuda and torch.cuda.is_current_stream_capturing()))
-    return (moe_grouped if grouped else moe_dense)(h, wts, gu_w, down_w, E, ff, ffs)
+    return (moe_grouped if grouped else moe_dense)(h, wts, gu_w, down_w, E, ff, ffs, act, gated)

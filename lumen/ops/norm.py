@@ -182,3 +182,47 @@ def group_rms_residual(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, groups
     call("sm_group_rms", DT[y.dtype], DT[cast if xb is not None else torch.float32], y,
          y.stride(0), w, x, xb, x.shape[1], x.shape[0], x.shape[1], groups, eps)
     return x, xb
+
+
+# ---- layer norm with a weight and no shift, fused with a scaled residual add -------------------
+# LN(x) = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w.  The fp32 residual stream takes a
+# sublayer's output multiplied by a constant, x += mult * y, and the same pass produces the next
+# sublayer's input LN(x) in the model dtype.  fp32 throughout; only a stored result is rounded.
+# (HIP: ``csrc/seqmix/layer_norm.hip``.)
+def weight_layer_norm_ref(x, w, eps, out_dtype=None):
+    xf = x.float()
+    d = xf - xf.mean(-1, keepdim=True)
+    y = d / torch.sqrt((d * d).mean(-1, keepdim=True) + eps) * w.float()
+    return y.to(out_dtype or x.dtype)
+
+
+def scaled_residual_layer_norm_ref(x, y, mult, w, eps, out_dtype=None):
+    if y is not None:
+        x.add_(y.float(), alpha=mult)
+    return x, (weight_layer_norm_ref(x, w, eps, out_dtype or x.dtype) if w is not None else None)
+
+
+def scaled_residual_layer_norm(x: torch.Tensor, y: Optional[torch.Tensor], mult: float,
+                               w: Optional[torch.Tensor], eps: float, out_dtype=None):
+    """The fp32 residual stream ``x`` [T, W] takes ``mult * y`` in place (``y`` None: nothing is
+    added) and -- fused, when ``w`` [W] (fp32) is given -- h = LN(x) * w is produced in
+    ``out_dtype``.  Returns (x, h or None)."""
+    from ._seqmix import DT, call, use_seqmix
+
+    if not use_seqmix(x):
+        return scaled_residual_layer_norm_ref(x, y, mult, w, eps, out_dtype)
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    assert y is None or (y.is_contiguous() and y.shape == x.shape)
+    assert w is None or (w.dtype == torch.float32 and w.is_contiguous())
+    if y is None and w is None:
+        return x, None
+    out_dtype = out_dtype or (y.dtype if y is not None else x.dtype)
+    h = torch.empty(x.shape, dtype=out_dtype, device=x.device) if w is not None else None
+    call("sm_layer_norm", DT[y.dtype] if y is not None else 0, DT[out_dtype], x, y, float(mult), w,
+         h, x.shape[0], x.shape[1], eps)
+    return x, h
+
+
+def weight_layer_norm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype=None) -> torch.Tensor:
+    """LN(x) * w of the fp32 rows ``x`` [T, W] in ``out_dtype``."""
+    return scaled_residual_layer_norm(x, None, 0.0, w, eps, out_dtype or x.dtype)[1]

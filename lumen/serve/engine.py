@@ -166,6 +166,12 @@ class LLMEngine:
             self.weights = WEIGHTS[model.config.arch](model, self.rank, self.tp)
         else:
             self.weights = ServeWeights(model, self.rank, self.tp)
+        limit = getattr(self.weights, "max_positions", None)
+        if limit is not None and cfg.max_model_len > limit:
+            # a learned position table ends there: no sequence may grow past its last row
+            from dataclasses import replace
+
+            cfg = self.cfg = replace(cfg, max_model_len=int(limit))
         if cfg.kv_cache_dtype not in ("auto", "fp8"):
             raise ValueError(f"kv_cache_dtype must be 'auto' or 'fp8', got {cfg.kv_cache_dtype}")
         self.kv_dtype = torch.float8_e4m3fn if cfg.kv_cache_dtype == "fp8" else dt

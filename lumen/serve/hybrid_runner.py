@@ -1,10 +1,11 @@
-"""Serving runner for stacks whose layers each name their own mixer (Gedatar, Dalavik): paged
-caches + per-sequence recurrent state.
+"""Serving runner for stacks whose layers each name their own mixer (Gedatar, Dalavik,
+Fanopel): paged caches + per-sequence recurrent state.
 
-Two families share the runner, the segments, the block manager and the hipGraph decode; each has
-its weights class (stacked projections, fp32 constants), its caches and its step function:
-Gedatar (``HybridWeights`` / ``HybridState`` / ``run_layers``, described next) and Dalavik
-(``DalavikWeights`` / ``DalavikState``, further down).
+Three families share the runner, the segments, the block manager and the hipGraph decode; each
+has its weights class (stacked projections, fp32 constants), its caches and its step function:
+Gedatar (``HybridWeights`` / ``HybridState`` / ``run_layers``, described next), Dalavik
+(``DalavikWeights`` / ``DalavikState``) and Fanopel (``FanopelWeights`` / ``FanopelState``),
+further down.
 
 One step function for prefill chunks, decode rows and mixtures of both.  The rows of a step are
 cut into segments (``ops.segments.SegBatch``: one per chunk, one per decode row); per layer
@@ -41,11 +42,12 @@ import torch.nn.functional as F
 from ..models.config import ModelConfig
 from ..models.gedatar import DELTA_DECAY, DELTA_KEY_EPS
 from ..ops.attention import (chunk_sink_attention, head_norm_write, latent_write, row_attention,
-                             transposed_values_ok, write_key_cache)
+                             row_norm_write, transposed_values_ok, write_key_cache)
 from ..ops.conv import dyt_canon
-from ..ops.embedding import gated_token_slice
-from ..ops.moe import gated_act, moe, route_topk
-from ..ops.norm import dyt, dyt_residual, group_rms_norm, group_rms_residual
+from ..ops.embedding import embed_positions, gated_token_slice
+from ..ops.moe import gated_act, moe, route_groups, route_topk
+from ..ops.norm import (dyt, dyt_residual, group_rms_norm, group_rms_residual,
+                        scaled_residual_layer_norm, weight_layer_norm)
 from ..ops.recurrent import delta_scan, token_shift, wkv_scan
 from ..ops.rope import rotate_interleaved_
 from ..ops.segments import SegBatch, whole_sequences
@@ -162,6 +164,9 @@ class HybridState:
 
 def key_bytes_per_token(cfg: ModelConfig, dtype_bytes: int = 2) -> int:
     """Bytes of paged cache one token takes over all layers."""
+    if cfg.arch == "fanopel":                  # normed keys + the keys as projected (the values)
+        return max(1, sum(2 * L["mixer"]["kv_heads"] * L["mixer"]["dim"]
+                          for L in cfg.layer_specs) * dtype_bytes)
     if cfg.arch == "dalavik":
         n = 0
         for L in cfg.layer_specs:
@@ -176,7 +181,7 @@ def key_bytes_per_token(cfg: ModelConfig, dtype_bytes: int = 2) -> int:
 
 
 def state_bytes_per_slot(cfg: ModelConfig) -> int:
-    if cfg.arch == "dalavik":
+    if cfg.arch in ("dalavik", "fanopel"):
         return 0
     n = 0
     for L in cfg.layer_specs:
@@ -427,7 +432,152 @@ def run_dalavik_layers(w: DalavikWeights, st: DalavikState, tokens: torch.Tensor
     return x
 
 
-WEIGHTS = {"gedatar": HybridWeights, "dalavik": DalavikWeights}
+# ---- Fanopel: gated window attention over keys-as-values + group-limited sigmoid routing ---------
+#
+#   x = embed[token] + pos[position]           fp32 stream (embed_positions); h = LN_1(x)
+#   attention
+#       z  = [W_q ; W_k ; W_g ; 0] h            one GEMM (rows padded to a multiple of 8 columns)
+#       q normed over the whole projection in place; k normed the same way into the key cache, k as
+#       projected into the value cache                                            (row_norm_write)
+#       o  = row_attention(soft cap, linear distance bias, window + kept first keys, sigmoid gate
+#            of z's gate columns on every head's output);  y = W_o o
+#   x += c y; h = LN_2(x)                       (scaled_residual_layer_norm, one pass)
+#   experts
+#       r  = route_groups(W_r h in fp32)        dense weights [T, E], zero off the chosen experts
+#       y  = [W_down_0 .. W_down_E-1] (relu(W_up h)^2 * r)     two stacked GEMMs, or per expert on
+#            its own rows for prefill-sized steps (ops.moe)
+#   x += c y; h = LN_1 of the next layer (or the final norm's weight after the last layer)
+#
+# fp32: the stream, every norm, the router, scores, softmax, the gate's sigmoid; model dtype: GEMMs
+# and what they store.  A sequence's whole memory is its cache blocks.
+@dataclass
+class FanopelLayerW:
+    m: dict                         # the mixer's sizes and constants
+    norm1: torch.Tensor
+    w: Dict[str, torch.Tensor] = field(default_factory=dict)
+    ff: Optional[dict] = None       # E, top, ff, up [E ff, W], down [W, E ff], router, correction...
+
+
+class FanopelWeights:
+    """Inference weights of a FanopelForCausalLM: q | k | gate stacked into one GEMM, the experts'
+    up projections stacked row-wise and their down projections side by side, norm weights, the
+    router, its correction and the distance-bias slopes in fp32."""
+
+    def __init__(self, model, tp_rank: int = 0, tp_size: int = 1):
+        if tp_size != 1:
+            raise NotImplementedError("Fanopel models are served at tensor-parallel size 1")
+        from ..models.fanopel import GROUP_RANK_TOP, ROUTE_SUM_EPS, head_slopes, router_groups
+
+        cfg: ModelConfig = model.config
+        self.cfg = cfg
+        t = model.tensor
+        f32 = lambda n: t(n).detach().float().contiguous()  # noqa: E731
+        self.dtype = t("embed").dtype
+        dev = t("embed").device
+        self.embed = t("embed").detach()
+        self.pos = t("pos").detach()
+        self.lm_head = t("head").detach()
+        self.final = f32("final.norm")
+        self.vocab_shard = cfg.vocab_size
+        self.max_positions = int(self.pos.shape[0])
+        self.mult = float(cfg.residual_mult)
+        self.layers: List[FanopelLayerW] = []
+        with torch.no_grad():
+            for i, spec in enumerate(cfg.layer_specs):
+                p, m = f"l{i}.", spec["mixer"]
+                x = p + "mix."
+                L = FanopelLayerW(m, f32(p + "norm1"))
+                H, G, D = m["heads"], m["kv_heads"], m["dim"]
+                W = cfg.hidden_size
+                rows = (H + G) * D + H
+                pad = -rows % 8                # the q / k / gate views keep 16-byte row strides
+                parts = [t(x + "q"), t(x + "k"), t(x + "g")]
+                if pad:
+                    parts.append(torch.zeros(pad, W, dtype=self.dtype, device=dev))
+                L.w["qkg"] = torch.cat(parts, 0).contiguous()
+                L.w["q.norm"], L.w["k.norm"] = f32(x + "q.norm"), f32(x + "k.norm")
+                L.w["slopes"] = head_slopes(H).to(dev)
+                L.w["o"] = t(x + "o").detach()
+                f = spec.get("mlp")
+                if f:
+                    y = p + "mlp."
+                    r = f["router"]
+                    E = r["experts"]
+                    n, keep = router_groups(f)
+                    L.ff = dict(E=E, top=int(r["top"]), ff=int(f["expert"]["ff"]), groups=n, keep=keep,
+                                scale=float(r.get("scale", 1.0)), sum_eps=ROUTE_SUM_EPS,
+                                rank_top=GROUP_RANK_TOP, norm=f32(p + "norm2"),
+                                up=torch.cat([t(y + f"e{e}.up") for e in range(E)], 0).contiguous(),
+                                down=torch.cat([t(y + f"e{e}.down") for e in range(E)], 1).contiguous(),
+                                router=f32(y + "router"), correction=f32(y + "correction"))
+                self.layers.append(L)
+
+    def new_state(self, slots: int, num_blocks: int, block_size: int, device):
+        return FanopelState(self, slots, num_blocks, block_size, device)
+
+    def run_layers(self, st, tokens, seg, observe=None) -> torch.Tensor:
+        return run_fanopel_layers(self, st, tokens, seg, observe)
+
+    def head(self, x: torch.Tensor) -> torch.Tensor:
+        return F.linear(weight_layer_norm(x, self.final, self.cfg.rms_norm_eps, self.dtype),
+                        self.lm_head)
+
+
+class FanopelState:
+    """Paged caches of a Fanopel model: per layer the normed keys (what the scores read) and the
+    keys as projected (the values), [blocks, block, kv_heads, dim] each.  No per-sequence state:
+    ``spare`` only names the slot number graph padding rows carry."""
+
+    def __init__(self, w: FanopelWeights, slots: int, num_blocks: int, block_size: int, device):
+        self.slots = slots
+        self.spare = slots
+        kw = dict(dtype=w.dtype, device=device)
+        shape = lambda m: (num_blocks, block_size, m["kv_heads"], m["dim"])  # noqa: E731
+        self.k = [torch.zeros(shape(L.m), **kw) for L in w.layers]
+        self.v = [torch.zeros(shape(L.m), **kw) for L in w.layers]
+
+
+def run_fanopel_layers(w: FanopelWeights, st: FanopelState, tokens: torch.Tensor, seg: SegBatch,
+                       observe=None) -> torch.Tensor:
+    """The step function: token ids [T] + their segments -> the fp32 residual stream [T, W]
+    after the last layer; the caches in ``st`` take the step's rows."""
+    cfg = w.cfg
+    dt = w.dtype
+    eps, c = cfg.rms_norm_eps, w.mult
+    T = tokens.shape[0]
+    x = embed_positions(tokens, seg.positions, w.embed, w.pos)
+    h = weight_layer_norm(x, w.layers[0].norm1, eps, dt)
+    n_layers = len(w.layers)
+    for i, L in enumerate(w.layers):
+        m = L.m
+        H, G, D = m["heads"], m["kv_heads"], m["dim"]
+        z = F.linear(h, L.w["qkg"])
+        row_norm_write(z, L.w["q.norm"], L.w["k.norm"], seg.cache_slots, st.k[i], st.v[i],
+                       H * D, G * D, eps)
+        o = torch.empty(T, H, D, dtype=dt, device=x.device)
+        mask = m["mask"]
+        row_attention(z[:, :H * D].view(T, H, D), None, st.k[i], st.v[i], D, o, seg, H, G,
+                      float(m["scale"]), float(m.get("softcap") or 0.0), slopes=L.w["slopes"],
+                      window=int(mask["size"]), keep_first=int(mask.get("keep_first", 0)),
+                      gate=z[:, (H + G) * D:(H + G) * D + H])
+        y = F.linear(o.view(T, H * D), L.w["o"])
+        nxt = w.layers[i + 1].norm1 if i + 1 < n_layers else None
+        f = L.ff
+        if f is None:
+            x, h = scaled_residual_layer_norm(x, y, c, nxt, eps, dt)
+        else:
+            x, h2 = scaled_residual_layer_norm(x, y, c, f["norm"], eps, dt)
+            # the router in fp32, on the (possibly 16-bit rounded) normed row
+            r = route_groups(h2.float() @ f["router"].t(), f["correction"], f["top"], f["groups"],
+                             f["keep"], f["scale"], f["sum_eps"], f["rank_top"])
+            y2 = moe(h2, r, f["up"], f["down"], f["E"], f["top"], f["ff"], 0, "relu2", gated=False)
+            x, h = scaled_residual_layer_norm(x, y2, c, nxt, eps, dt)
+        if observe is not None:
+            observe(i, x)
+    return x
+
+
+WEIGHTS = {"gedatar": HybridWeights, "dalavik": DalavikWeights, "fanopel": FanopelWeights}
 
 
 class HybridRunner(ModelRunner):
