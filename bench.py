@@ -494,7 +494,8 @@ def main():
                     help="instead of the default workload: prefill / decode throughput of a "
                          "per-layer-mixer design (--hybrid_family) beside Llama at equal size, "
                          "one GPU (lumen/bench/hybrid_bench.py)")
-    ap.add_argument("--hybrid_family", default="gedatar", choices=["gedatar", "dalavik"])
+    ap.add_argument("--hybrid_family", default="gedatar",
+                    choices=["gedatar", "dalavik", "fanopel"])
     ap.add_argument("--hybrid_widths", default="2048,4096")
     ap.add_argument("--hybrid_batch", default="8,64", help="sequences per step (comma list)")
     ap.add_argument("--hybrid_prompt", type=int, default=512)

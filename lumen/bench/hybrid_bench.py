@@ -1,7 +1,9 @@
-"""Prefill / decode throughput of a per-layer-mixer design (Gedatar, Dalavik) beside Llama at
-equal size.
+"""Prefill / decode throughput of a per-layer-mixer design (Gedatar, Dalavik, Fanopel) beside
+Llama at equal size.
 
-``python bench.py --hybrid [--hybrid_family dalavik]`` (one GPU).  Both models get random
+``python bench.py --hybrid [--hybrid_family dalavik|fanopel]`` (one GPU).  Fanopel also runs
+beside the closest design the framework already had: a Gedatar stack of attention layers (keys
+as values) with routed experts of the same shapes.  Both models get random
 weights of layer shapes that resemble real models (width 2048 / 4096, head size 128 / 64, FFN 2.75 x width, vocab 32000), the
 same depth, and run the same forced-token workload through the serving engine
 (``lumen.serve.trace.TraceReplay``: the engine's input builder, block manager, state slots,
@@ -71,6 +73,44 @@ def dalavik_config(width: int, depth_groups: int = 1):
                        token_side_dim=128, intermediate_size=0, num_attention_heads=0,
                        num_key_value_heads=0, max_position_embeddings=1 << 20, eos_token_id=-1,
                        tie_word_embeddings=True, name=f"dalavik-w{W}", layer_specs=layers)
+
+
+def fanopel_config(width: int, depth: int = 4):
+    """Gated window attention (heads of 128, one key head per four query heads, window 1024 + 4
+    kept tokens, soft cap 30) and 16 routed experts of FFN width 2.75 / 4 x model width in 4 groups
+    of which 2 are kept, top 4: the active FFN width equals the dense 2.75 x width."""
+    from ..models.config import ModelConfig
+
+    W = width
+    layer = {"type": "attention",
+             "mixer": {"heads": W // 128, "kv_heads": max(1, W // 512), "dim": 128, "vdim": 128,
+                       "scale": 128 ** -0.5, "softcap": 30.0,
+                       "mask": {"size": 1024, "keep_first": 4}},
+             "mlp": {"kind": "moe", "expert": {"ff": int(2.75 * W) // 4},
+                     "router": {"experts": 16, "top": 4, "scale": 2.0,
+                                "groups": {"count": 4, "keep": 2}}}}
+    return ModelConfig(arch="fanopel", vocab_size=32000, hidden_size=W, num_hidden_layers=depth,
+                       rms_norm_eps=1e-6, residual_mult=0.5, intermediate_size=0,
+                       num_attention_heads=0, num_key_value_heads=0, max_position_embeddings=4096,
+                       eos_token_id=-1, name=f"fanopel-w{W}", layer_specs=[layer] * depth)
+
+
+def gedatar_attention_moe_config(width: int, depth: int = 4):
+    """The closest older design at Fanopel's shapes: Gedatar attention layers (keys as values,
+    chunk mask of 1024) with 16 gated experts of the same FFN width, top 4, no shared expert."""
+    from ..models.config import ModelConfig
+
+    W = width
+    layer = {"type": "attention",
+             "mixer": {"heads": W // 128, "kv_heads": max(1, W // 512), "dim": 128, "vdim": 128,
+                       "scale": 0.09, "mask": {"size": 1024}},
+             "mlp": {"kind": "moe", "router": {"experts": 16, "top": 4},
+                     "expert": {"ff": int(2.75 * W) // 4}}}
+    return ModelConfig(arch="gedatar", vocab_size=32000, hidden_size=W, num_hidden_layers=depth,
+                       rms_norm_eps=1e-6, canon_taps=4, intermediate_size=0,
+                       num_attention_heads=0, num_key_value_heads=0,
+                       max_position_embeddings=1 << 20, eos_token_id=-1,
+                       name=f"gedatar-attnmoe-w{W}", layer_specs=[layer] * depth)
 
 
 def llama_config(width: int, layers: int):
@@ -147,10 +187,13 @@ def run_hybrid_bench(args) -> list:
     assert native() is not None, native_error()
     rows = []
     family = getattr(args, "hybrid_family", "gedatar")
-    make = {"gedatar": gedatar_config, "dalavik": dalavik_config}[family]
+    make = {"gedatar": gedatar_config, "dalavik": dalavik_config, "fanopel": fanopel_config}[family]
     for width in [int(w) for w in str(args.hybrid_widths).split(",")]:
         gcfg = make(width)
-        for cfg in (gcfg, llama_config(width, gcfg.num_hidden_layers)):
+        beside = [llama_config(width, gcfg.num_hidden_layers)]
+        if family == "fanopel":
+            beside.insert(0, gedatar_attention_moe_config(width, gcfg.num_hidden_layers))
+        for cfg in [gcfg] + beside:
             for batch in [int(b) for b in str(args.hybrid_batch).split(",")]:
                 r = run_one(cfg, batch, args.hybrid_prompt, args.hybrid_decode_steps, 3, dev)
                 r["width"] = width
@@ -158,13 +201,18 @@ def run_hybrid_bench(args) -> list:
                 print(json.dumps(r), flush=True)
     by = {(r["width"], r["batch"], r["model"].split("-")[0]): r for r in rows}
     summ = []
-    for (w, b, kind), r in by.items():
+    for (w, b, kind), r in list(by.items()):
         if kind != family:
             continue
         ll = by[(w, b, "llama")]
-        summ.append({"width": w, "batch": b,
-                     "prefill_vs_llama": round(r["prefill_tok_s"] / ll["prefill_tok_s"], 3),
-                     "decode_vs_llama": round(r["decode_tok_s"] / ll["decode_tok_s"], 3)})
+        row = {"width": w, "batch": b,
+               "prefill_vs_llama": round(r["prefill_tok_s"] / ll["prefill_tok_s"], 3),
+               "decode_vs_llama": round(r["decode_tok_s"] / ll["decode_tok_s"], 3)}
+        if family == "fanopel":
+            gd = by[(w, b, "gedatar")]
+            row["prefill_vs_gedatar"] = round(r["prefill_tok_s"] / gd["prefill_tok_s"], 3)
+            row["decode_vs_gedatar"] = round(r["decode_tok_s"] / gd["decode_tok_s"], 3)
+        summ.append(row)
     metric = "hybrid" if family == "gedatar" else family
     print(json.dumps({"metric": f"{metric}_vs_llama_tokens_per_s", "dtype": "bf16",
                       "data": "synthetic", "rows": summ}), flush=True)

@@ -365,10 +365,12 @@ HUB_ALIASES = {
 
 def get_config(name_or_path: str) -> ModelConfig:
     """Resolve a preset name, an HF hub id (offline alias) or a local HF checkpoint dir."""
-    if name_or_path in PRESETS:
-        return ModelConfig(**PRESETS[name_or_path])
     if name_or_path in HUB_ALIASES:
-        return ModelConfig(**PRESETS[HUB_ALIASES[name_or_path]])
+        name_or_path = HUB_ALIASES[name_or_path]
+    if name_or_path in PRESETS:
+        import copy
+
+        return ModelConfig(**copy.deepcopy(PRESETS[name_or_path]))   # layer lists are the caller's
     if os.path.isdir(name_or_path):
         cfg_path = os.path.join(name_or_path, "config.json")
         with open(cfg_path) as f:
