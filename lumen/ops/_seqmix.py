@@ -41,6 +41,7 @@ SIGNATURES = {
     "sm_latent_attn": "i" "plli" "plli" "pl" "pi" "pll" "pi" "pp" "iii" "fffi" "ppp" "ipp",
     "sm_row_attn": "i" "plli" "plli" "pl" "pli" "pll" "pi" "pp" "iiiii" "fffi" "pppp" "piipl"
                    "ipp",
+    "sm_win_attn_tiles": "iplppppl" "pi" "pi" "pp" "iiii" "ff" "p" "iii",
     "sm_row_norm_write": "iplpppppiiif",
     "sm_layer_norm": "iippfppiif",
     "sm_embed_pos": "ipppppiiii",
@@ -66,6 +67,8 @@ def _load():
             fn.restype = ctypes.c_int
         lib.sm_chunk_attn_tiles_ok.argtypes = [ctypes.c_int, ctypes.c_int]
         lib.sm_chunk_attn_tiles_ok.restype = ctypes.c_int
+        lib.sm_win_attn_tiles_ok.argtypes = [ctypes.c_int, ctypes.c_int]
+        lib.sm_win_attn_tiles_ok.restype = ctypes.c_int
         lib.sm_row_attn_lds.argtypes = [ctypes.c_int, ctypes.c_int]
         lib.sm_row_attn_lds.restype = ctypes.c_int
         lib.sm_latent_attn_ok.argtypes = [ctypes.c_int] * 5
@@ -97,6 +100,12 @@ DT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 def tiles_ok(dt: int, D: int) -> bool:
     """Does the matrix-core prefill attention have a kernel for this dtype code / head size?"""
     return bool(_load().sm_chunk_attn_tiles_ok(dt, D))
+
+
+def win_tiles_ok(dt: int, D: int) -> bool:
+    """Does the matrix-core prefill attention over paged key and value caches have a kernel for
+    this dtype code / head size?"""
+    return bool(_load().sm_win_attn_tiles_ok(dt, D))
 
 
 def row_attn_lds(HB: int, Dk: int) -> int:

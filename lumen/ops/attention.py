@@ -802,7 +802,7 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
     head h's output is multiplied by sigmoid(gate[t, h]).  ``vt`` [blocks, Dv, block]: a per-block transposed copy of the
     values (``latent_write`` keeps one); with it, one key/value head, values that are a prefix of
     the key rows and a 16-bit dtype, the whole kernel runs on the matrix cores."""
-    from ._seqmix import DT, call, latent_attn_ok, use_seqmix
+    from ._seqmix import DT, call, latent_attn_ok, use_seqmix, win_tiles_ok
 
     T, _, D1 = q1.shape
     D2 = q2.shape[2] if q2 is not None else 0
@@ -846,6 +846,25 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
              seg.tables, seg.tables.shape[1], seg.row_seg, seg.positions, T, H, bs,
              scale, float(softcap or 0.0), coef, every, r1, r2, sink, nsplit, ws_ml, ws_o)
         return out
+    # a step's prompt portions: tiles of consecutive rows of one segment on the matrix cores, when
+    # nothing needs all heads of a (row, key) pair at once and the kernel has the head size; the
+    # decoded rows after them (and every other case) take the row kernel below
+    Tp = 0
+    if (seg.q_tiles is not None and seg.tile_rows > 0 and q2 is None and talk is None
+            and sink is None and r1 is None and q_temp is None and vcache is not kcache
+            and D1 == Dv and krow == G * D1 and vrow == G * Dv and win_tiles_ok(DT[q1.dtype], D1)
+            and q1.stride(1) == D1 and q1.stride(0) % 8 == 0 and q1.data_ptr() % 16 == 0
+            and out.stride(1) == Dv and out.stride(0) == H * Dv and out.data_ptr() % 8 == 0):
+        Tp = seg.tile_rows
+        call("sm_win_attn_tiles", DT[q1.dtype], q1, q1.stride(0), kcache, vcache, out, gate,
+             gate.stride(0) if gate is not None else 0, seg.tables, seg.tables.shape[1],
+             seg.q_tiles, seg.q_tiles.shape[0], seg.cu, seg.start, H, G, D1, bs, scale,
+             float(softcap or 0.0), slopes, window, keep_first, seg.tile_size)
+        if Tp >= T:
+            return out
+        q1, out, T = q1[Tp:], out[Tp:], T - Tp
+        gate = gate[Tp:] if gate is not None else None
+    row_seg, positions = seg.row_seg[Tp:], seg.positions[Tp:]
     HB = _heads_per_block(H, Dk, talk is not None)
     # few rows (decoding): deal a row's 64-key tiles out to several workgroups so that ~2 per CU
     # run; the count depends on the step's size only, never on device data (graph capture)
@@ -863,7 +882,7 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
     call("sm_row_attn", DT[q1.dtype], q1, q1.stride(0), q1.stride(1), D1,
          q2, q2.stride(0) if q2 is not None else 0, q2.stride(1) if q2 is not None else 0, D2,
          kcache, krow, vcache, vrow, Dv, out, out.stride(0), out.stride(1),
-         seg.tables, seg.tables.shape[1], seg.row_seg, seg.positions, T, H, G, HB,
+         seg.tables, seg.tables.shape[1], row_seg, positions, T, H, G, HB,
          kcache.shape[1], scale, float(softcap or 0.0), coef, every, r1, r2, talk, sink,
          slopes, window, keep_first, gate, gate.stride(0) if gate is not None else 0,
          nsplit, ws_ml, ws_o)

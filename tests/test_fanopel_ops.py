@@ -161,9 +161,73 @@ def test_row_attention_window_bias_gate(device, dtype, H, G, D, bs, window, keep
         at += n
 
 
+def tiled_segments(spans, n_prompt, tables, device, rows):
+    """As ``segments``, with the first ``n_prompt`` spans cut into tiles of ``rows`` rows: the
+    form in which the engine hands a step's prompt portions to the matrix-core kernel."""
+    from lumen.ops.segments import tile_list
+
+    seg = segments(spans, tables, device)
+    cu = seg.cu.tolist()
+    seg.q_tiles = torch.tensor(tile_list(cu, n_prompt, rows), dtype=torch.int32,
+                               device=device).view(-1, 2)
+    seg.tile_rows, seg.tile_size = cu[n_prompt], rows
+    return seg
+
+
+TILE_SPANS = [(0, 0, 20), (2, 60, 39), (3, 310, 390), (1, 100, 33), (4, 0, 1), (5, 7, 2),
+              (6, 0, 300),                                         # prompt portions ...
+              (7, 130, 1), (8, 299, 1)]                            # ... then decoded rows
+TILE_LENS = [20, 133, 99, 700, 1, 9, 300, 131, 300]             # by sequence
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows", [64, 128])
+@pytest.mark.parametrize("H,G,D,bs,window,keep", [
+    (4, 2, 32, 8, 21, 3), (3, 3, 64, 16, 70, 1), (4, 1, 96, 16, 136, 5), (8, 2, 128, 16, 64, 0),
+    (2, 2, 128, 16, 65, 64), (2, 1, 192, 16, 130, 70), (2, 2, 256, 32, 1, 2), (6, 3, 64, 4, 1000, 4),
+    (2, 1, 64, 16, 0, 0), (2, 2, 32, 16, 33, 31), (2, 2, 32, 16, 32, 33), (4, 4, 64, 16, 300, 200)])
+def test_prompt_portions_on_the_matrix_cores(dtype, rows, H, G, D, bs, window, keep):
+    """The tiled kernel takes a step's prompt portions (whole prompts, portions that start far
+    into a sequence, portions of one and two rows, a portion longer than the window so that key
+    tiles between the kept keys and the window are skipped), the row kernel the decoded rows
+    behind them; both against the dense formula.  window 0: plain causal attention."""
+    device = "cuda"
+    ks = [rnd(n, G * D, seed=20 + i, dtype=dtype) for i, n in enumerate(TILE_LENS)]
+    vs = [rnd(n, G * D, seed=40 + i, dtype=dtype) for i, n in enumerate(TILE_LENS)]
+    nb = sum((n + bs - 1) // bs for n in TILE_LENS) + 3
+    kc, tb = paged(ks, bs, nb, G * D, dtype, device, 1)
+    vc, _ = paged(vs, bs, nb, G * D, dtype, device, 1)
+    seg = tiled_segments(TILE_SPANS, 7, tb, device, rows)
+    T = seg.T
+    pad = -(H * D + H) % 8
+    z = rnd(T, H * D + H + pad, seed=60, dtype=dtype, device=device)
+    q, gate = z[:, :H * D].view(T, H, D), z[:, H * D:H * D + H]
+    slopes = torch.tensor([2.0 ** (-6.0 * (h + 1) / H) for h in range(H)], device=device)
+    out = torch.zeros(T, H, D, dtype=dtype, device=device)
+    sc = 0.3 * (32.0 / D) ** 0.5
+    row_attention(q, None, kc.view(nb, bs, G, D), vc.view(nb, bs, G, D), D, out, seg, H, G, sc,
+                  softcap=5.0, slopes=slopes, window=window, keep_first=keep, gate=gate)
+    hg = torch.arange(H) // (H // G)
+    at = 0
+    for s, p0, n in TILE_SPANS:
+        pos = torch.arange(p0, p0 + n)
+        want = dense_window_attention(q[at:at + n].cpu(), ks[s][:p0 + n].view(-1, G, D),
+                                      vs[s][:p0 + n].view(-1, G, D), pos, hg, sc, 5.0,
+                                      slopes.cpu(), window, keep, gate[at:at + n].cpu())
+        close(out[at:at + n], want, dtype, scale=1.0)
+        at += n
+    # the same rows through the row kernel alone: the two kernels agree to rounding
+    seg.q_tiles, seg.tile_rows = None, 0
+    out2 = torch.zeros_like(out)
+    row_attention(q, None, kc.view(nb, bs, G, D), vc.view(nb, bs, G, D), D, out2, seg, H, G, sc,
+                  softcap=5.0, slopes=slopes, window=window, keep_first=keep, gate=gate)
+    close(out, out2.cpu().to(F64), dtype, scale=1.0)
+
+
 @pytest.mark.parametrize("device,dtype", CASES)
 @pytest.mark.parametrize("window,keep", [(136, 4), (64, 1), (65, 0), (200, 64), (30, 65), (1, 1)])
-@pytest.mark.parametrize("rows", ["decoded", "prompt"])
+@pytest.mark.parametrize("rows", ["decoded", "prompt", "tiled"])
 def test_window_and_kept_edges(device, dtype, window, keep, rows):
     """One key carries a spike the query is aligned with.  Placed at the last position inside the
     window, at the first one outside it, at the last kept position and at the first one behind the
@@ -190,7 +254,8 @@ def test_window_and_kept_edges(device, dtype, window, keep, rows):
         kc, tb = paged([k.to(dtype)], bs, 50, D, dtype, device, 3)
         vc, _ = paged([v.to(dtype)], bs, 50, D, dtype, device, 3)
         spans = [(0, p, 1)] if rows == "decoded" else [(0, p - 30, 31)]
-        seg = segments(spans, tb, device)
+        seg = (tiled_segments(spans, 1, tb, device, 128) if rows == "tiled"
+               else segments(spans, tb, device))
         q = (8.0 * d).to(dtype).to(device).expand(seg.T, H, D).contiguous()
         out = torch.zeros(seg.T, H, D, dtype=dtype, device=device)
         row_attention(q, None, kc.view(50, bs, 1, D), vc.view(50, bs, 1, D), D, out, seg, H, 1, 1.0,
