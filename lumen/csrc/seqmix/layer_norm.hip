@@ -17,54 +17,91 @@ namespace {
 
 constexpr int kThreads = 256;
 
-template <typename TY, typename TO>
+// VEC: four consecutive entries per thread and step (16 bytes of fp32, 8 bytes of a 16-bit type);
+// the launcher picks it when W is a multiple of 4 and the pointers are aligned for it
+template <typename TY, typename TO, bool VEC>
 __global__ void __launch_bounds__(kThreads)
 layer_norm_kernel(float* __restrict__ x, const TY* __restrict__ y, float mult,
                   const float* __restrict__ w, TO* __restrict__ out, int W, float eps) {
   extern __shared__ float s_row[];
   __shared__ float s_red[kThreads / 64];
+  constexpr int V = VEC ? 4 : 1;
   const long long base = (long long)blockIdx.x * W;
   float sum = 0.f;
-  for (int c = threadIdx.x; c < W; c += kThreads) {
-    float v = x[base + c];
-    if (y != nullptr) {
-      v += mult * to_f32(y[base + c]);
-      x[base + c] = v;
+  for (int c = threadIdx.x * V; c < W; c += kThreads * V) {
+    if constexpr (VEC) {
+      float v[4];
+      load4<float>(x + base + c, v);
+      if (y != nullptr) {
+        float yv[4];
+        load4<TY>(y + base + c, yv);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += mult * yv[e];
+        store4<float>(x + base + c, v);
+      }
+      store4<float>(s_row + c, v);
+      sum += (v[0] + v[1]) + (v[2] + v[3]);
+    } else {
+      float v = x[base + c];
+      if (y != nullptr) {
+        v += mult * to_f32(y[base + c]);
+        x[base + c] = v;
+      }
+      s_row[c] = v;
+      sum += v;
     }
-    s_row[c] = v;
-    sum += v;
   }
   if (w == nullptr) return;
   const float mean = block_sum<kThreads>(sum, s_red) / (float)W;
   float sq = 0.f;
-  for (int c = threadIdx.x; c < W; c += kThreads) {       // a thread re-reads its own entries
-    const float d = s_row[c] - mean;
-    sq += d * d;
+  for (int c = threadIdx.x * V; c < W; c += kThreads * V) {   // a thread re-reads its own entries
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const float d = s_row[c + e] - mean;
+      sq += d * d;
+    }
   }
   const float inv = 1.f / sqrtf(block_sum<kThreads>(sq, s_red) / (float)W + eps);
-  for (int c = threadIdx.x; c < W; c += kThreads)
-    out[base + c] = from_f32<TO>((s_row[c] - mean) * inv * w[c]);
+  for (int c = threadIdx.x * V; c < W; c += kThreads * V) {
+    if constexpr (VEC) {
+      float v[4], ww[4];
+      load4<float>(s_row + c, v);
+      load4<float>(w + c, ww);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = (v[e] - mean) * inv * ww[e];
+      store4<TO>(out + base + c, v);
+    } else {
+      out[base + c] = from_f32<TO>((s_row[c] - mean) * inv * w[c]);
+    }
+  }
 }
 
-template <typename T>
-__global__ void embed_pos_kernel(const T* __restrict__ table, const T* __restrict__ pos_table,
-                                 const long long* __restrict__ tokens,
-                                 const int* __restrict__ positions, float* __restrict__ out,
-                                 long long n, int W, int V, int P) {
-  for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < n;
-       i += (long long)gridDim.x * blockDim.x) {
-    const long long t = i / W;
-    const int c = (int)(i % W);
+// one workgroup per row; 8 entries per thread and step when W is a multiple of 8
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(256)
+embed_pos_kernel(const T* __restrict__ table, const T* __restrict__ pos_table,
+                 const long long* __restrict__ tokens, const int* __restrict__ positions,
+                 float* __restrict__ out, int Tn, int W, int V, int P) {
+  for (int t = blockIdx.x; t < Tn; t += gridDim.x) {
     // the host bounds both indices; a stray one reads the table's edge instead of faulting
     const long long tok = min(max(tokens[t], 0ll), (long long)V - 1);
     const int p = min(max(positions[t], 0), P - 1);
-    out[i] = to_f32(table[tok * W + c]) + to_f32(pos_table[(long long)p * W + c]);
+    const T* a = table + tok * W;
+    const T* b = pos_table + (long long)p * W;
+    float* o = out + (long long)t * W;
+    if constexpr (VEC) {
+      for (int c = 8 * threadIdx.x; c < W; c += 8 * 256) {
+        float u[8], v[8];
+        load8<T>(a + c, u);
+        load8<T>(b + c, v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) u[e] += v[e];
+        store8<float>(o + c, u);
+      }
+    } else {
+      for (int c = threadIdx.x; c < W; c += 256) o[c] = to_f32(a[c]) + to_f32(b[c]);
+    }
   }
-}
-
-inline int grid_for(long long n, int block = 256) {
-  const long long g = (n + block - 1) / block;
-  return (int)(g < 1 ? 1 : g > 65535 ? 65535 : g);
 }
 
 }  // namespace
@@ -78,19 +115,24 @@ hipError_t sm_layer_norm(int dt_y, int dt_out, float* x, const void* y, float mu
   if (rows == 0 || (!y && !w)) return hipSuccess;
   if (W < 1 || (size_t)W * sizeof(float) > 65536 - 64 || (w && !out)) return hipErrorInvalidValue;
   const size_t lds = (size_t)W * sizeof(float);
-#define CALL_O(TO)                                                                              \
+  const bool vec = W % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0 &&
+                   (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0;
+#define CALL_Y(TY, TO)                                                                          \
   {                                                                                             \
-    if (dt_y == kF32)                                                                           \
-      layer_norm_kernel<float, TO><<<rows, kThreads, lds, st>>>(x, (const float*)y, mult, w,    \
-                                                                (TO*)out, W, eps);              \
-    else if (dt_y == kBF16)                                                                     \
-      layer_norm_kernel<bf16, TO><<<rows, kThreads, lds, st>>>(x, (const bf16*)y, mult, w,      \
-                                                               (TO*)out, W, eps);               \
-    else if (dt_y == kF16)                                                                      \
-      layer_norm_kernel<fp16, TO><<<rows, kThreads, lds, st>>>(x, (const fp16*)y, mult, w,      \
-                                                               (TO*)out, W, eps);               \
-    else return hipErrorInvalidValue;                                                           \
-    break;                                                                                      \
+    if (vec)                                                                                    \
+      layer_norm_kernel<TY, TO, true><<<rows, kThreads, lds, st>>>(x, (const TY*)y, mult, w,    \
+                                                                   (TO*)out, W, eps);           \
+    else                                                                                        \
+      layer_norm_kernel<TY, TO, false><<<rows, kThreads, lds, st>>>(x, (const TY*)y, mult, w,   \
+                                                                    (TO*)out, W, eps);          \
+  }
+#define CALL_O(TO)                                    \
+  {                                                   \
+    if (dt_y == kF32) CALL_Y(float, TO)               \
+    else if (dt_y == kBF16) CALL_Y(bf16, TO)          \
+    else if (dt_y == kF16) CALL_Y(fp16, TO)           \
+    else return hipErrorInvalidValue;                 \
+    break;                                            \
   }
   switch (dt_out) {
     case kF32: CALL_O(float)
@@ -99,16 +141,23 @@ hipError_t sm_layer_norm(int dt_y, int dt_out, float* x, const void* y, float mu
     default: return hipErrorInvalidValue;
   }
 #undef CALL_O
+#undef CALL_Y
   return hipGetLastError();
 }
 
 hipError_t sm_embed_pos(int dt, const void* table, const void* pos_table, const long long* tokens,
                         const int* positions, float* out, int T, int W, int V, int P,
                         hipStream_t st) {
-  const long long n = (long long)T * W;
-  if (n == 0) return hipSuccess;
+  if ((long long)T * W == 0) return hipSuccess;
   if (V < 1 || P < 1) return hipErrorInvalidValue;
-#define CALL(TT) embed_pos_kernel<TT><<<grid_for(n), 256, 0, st>>>((const TT*)table, (const TT*)pos_table, tokens, positions, out, n, W, V, P)
+  const bool vec = W % 8 == 0 && (uintptr_t)table % 16 == 0 && (uintptr_t)pos_table % 16 == 0 &&
+                   (uintptr_t)out % 16 == 0;
+  const int grid = T < 65535 ? T : 65535;
+#define CALL(TT)                                                                                  \
+  if (vec) embed_pos_kernel<TT, true><<<grid, 256, 0, st>>>((const TT*)table, (const TT*)pos_table, \
+                                                           tokens, positions, out, T, W, V, P);  \
+  else embed_pos_kernel<TT, false><<<grid, 256, 0, st>>>((const TT*)table, (const TT*)pos_table,  \
+                                                         tokens, positions, out, T, W, V, P)
   SM_DISPATCH(dt, CALL)
 #undef CALL
   return hipGetLastError();

@@ -194,25 +194,40 @@ head_norm_write_kernel(T* __restrict__ qkv, long long ld, const float* __restric
 
 // One workgroup per row: the sums of squares of the query part (HD entries) and of the key part
 // (GD entries) are reduced over the four waves in a fixed order, then q is normed in place and the
-// key goes to both caches.
-template <typename T>
+// key goes to both caches.  VEC: 8 entries (16 bytes of a 16-bit type) per thread and step.
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(64 * kWaves)
 row_norm_write_kernel(T* __restrict__ qk, long long ld, const float* __restrict__ wq,
                       const float* __restrict__ wk, const long long* __restrict__ slots,
                       T* __restrict__ kcache, T* __restrict__ vcache, int HD, int GD, float eps) {
   __shared__ float s_red[2][kWaves];
+  constexpr int V = VEC ? 8 : 1, NT = 64 * kWaves;
   const int t = blockIdx.x, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const long long s = slots[t];
   T* q = qk + (long long)t * ld;
   const T* k = q + HD;
   float sq = 0.f, sk = 0.f;
-  for (int c = threadIdx.x; c < HD; c += 64 * kWaves) {
-    const float v = to_f32(q[c]);
-    sq += v * v;
+  for (int c = threadIdx.x * V; c < HD; c += NT * V) {
+    if constexpr (VEC) {
+      float v[8];
+      load8<T>(q + c, v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sq += v[e] * v[e];
+    } else {
+      const float v = to_f32(q[c]);
+      sq += v * v;
+    }
   }
-  for (int c = threadIdx.x; c < GD; c += 64 * kWaves) {
-    const float v = to_f32(k[c]);
-    sk += v * v;
+  for (int c = threadIdx.x * V; c < GD; c += NT * V) {
+    if constexpr (VEC) {
+      float v[8];
+      load8<T>(k + c, v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sk += v[e] * v[e];
+    } else {
+      const float v = to_f32(k[c]);
+      sk += v * v;
+    }
   }
   sq = wave_sum(sq);
   sk = wave_sum(sk);
@@ -227,13 +242,34 @@ row_norm_write_kernel(T* __restrict__ qk, long long ld, const float* __restrict_
   if (s >= 0) {
     T* kd = kcache + s * GD;
     T* vd = vcache + s * GD;
-    for (int c = threadIdx.x; c < GD; c += 64 * kWaves) {
-      const T raw = k[c];
-      vd[c] = raw;
-      kd[c] = from_f32<T>(to_f32(raw) * ik * wk[c]);
+    for (int c = threadIdx.x * V; c < GD; c += NT * V) {
+      if constexpr (VEC) {
+        *reinterpret_cast<uint4*>(vd + c) = *reinterpret_cast<const uint4*>(k + c);
+        float v[8], ww[8];
+        load8<T>(k + c, v);
+        load8<float>(wk + c, ww);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = v[e] * ik * ww[e];
+        store8<T>(kd + c, v);
+      } else {
+        const T raw = k[c];
+        vd[c] = raw;
+        kd[c] = from_f32<T>(to_f32(raw) * ik * wk[c]);
+      }
     }
   }
-  for (int c = threadIdx.x; c < HD; c += 64 * kWaves) q[c] = from_f32<T>(to_f32(q[c]) * iq * wq[c]);
+  for (int c = threadIdx.x * V; c < HD; c += NT * V) {
+    if constexpr (VEC) {
+      float v[8], ww[8];
+      load8<T>(q + c, v);
+      load8<float>(wq + c, ww);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = v[e] * iq * ww[e];
+      store8<T>(q + c, v);
+    } else {
+      q[c] = from_f32<T>(to_f32(q[c]) * iq * wq[c]);
+    }
+  }
 }
 
 // Workgroups are handed to the 8 XCDs round-robin in launch order, and every XCD has an L2 of its
@@ -903,7 +939,15 @@ hipError_t sm_row_norm_write(int dt, void* qk, long long ld, const float* wq, co
                              int GD, float eps, hipStream_t st) {
   if (T == 0) return hipSuccess;
   if (HD < 1 || GD < 1 || ld < HD + GD) return hipErrorInvalidValue;
-#define CALL(TT) row_norm_write_kernel<TT><<<T, 64 * kWaves, 0, st>>>((TT*)qk, ld, wq, wk, slots, (TT*)kcache, (TT*)vcache, HD, GD, eps)
+  // 16-byte accesses: 16-bit dtypes, every part a multiple of 8 entries, aligned bases
+  const bool vec = dt != kF32 && HD % 8 == 0 && GD % 8 == 0 && ld % 8 == 0 &&
+                   (uintptr_t)qk % 16 == 0 && (uintptr_t)kcache % 16 == 0 &&
+                   (uintptr_t)vcache % 16 == 0 && (uintptr_t)wq % 16 == 0 && (uintptr_t)wk % 16 == 0;
+#define CALL(TT)                                                                                \
+  if (vec) row_norm_write_kernel<TT, true><<<T, 64 * kWaves, 0, st>>>(                          \
+      (TT*)qk, ld, wq, wk, slots, (TT*)kcache, (TT*)vcache, HD, GD, eps);                       \
+  else row_norm_write_kernel<TT, false><<<T, 64 * kWaves, 0, st>>>(                             \
+      (TT*)qk, ld, wq, wk, slots, (TT*)kcache, (TT*)vcache, HD, GD, eps)
   SM_DISPATCH(dt, CALL)
 #undef CALL
   return hipGetLastError();
