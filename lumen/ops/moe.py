@@ -48,6 +48,16 @@ def route_topk(z: torch.Tensor, top: int) -> torch.Tensor:
     return out
 
 
+def router_logits(h: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """fp32 router logits h [T, W] @ w [E, W]^T for h and w in the model dtype.  16-bit values
+    multiply exactly in fp32, so on the GPU the product runs on the matrix cores with fp32
+    accumulation and an fp32 result -- the arithmetic of an fp32 GEMM on the widened operands
+    without the pass that widens them."""
+    if h.is_cuda and h.dtype == w.dtype and h.dtype in (torch.bfloat16, torch.float16):
+        return torch.mm(h, w.t(), out_dtype=torch.float32)
+    return h.float() @ w.float().t()
+
+
 def route_groups_ref(z, correction, top, n_groups, keep, scale, sum_eps=1e-20, rank_top=2):
     T, E = z.shape
     s = torch.sigmoid(z.float())

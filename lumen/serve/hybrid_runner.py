@@ -45,7 +45,7 @@ from ..ops.attention import (chunk_sink_attention, head_norm_write, latent_write
                              row_norm_write, transposed_values_ok, write_key_cache)
 from ..ops.conv import dyt_canon
 from ..ops.embedding import embed_positions, gated_token_slice
-from ..ops.moe import gated_act, moe, route_groups, route_topk
+from ..ops.moe import gated_act, moe, route_groups, route_topk, router_logits
 from ..ops.norm import (dyt, dyt_residual, group_rms_norm, group_rms_residual,
                         scaled_residual_layer_norm, weight_layer_norm)
 from ..ops.recurrent import delta_scan, token_shift, wkv_scan
@@ -444,6 +444,7 @@ def run_dalavik_layers(w: DalavikWeights, st: DalavikState, tokens: torch.Tensor
 #   x += c y; h = LN_2(x)                       (scaled_residual_layer_norm, one pass)
 #   experts
 #       r  = route_groups(W_r h in fp32)        dense weights [T, E], zero off the chosen experts
+#            (router_logits: exact 16-bit products, fp32 accumulation and result)
 #       y  = [W_down_0 .. W_down_E-1] (relu(W_up h)^2 * r)     two stacked GEMMs, or per expert on
 #            its own rows for prefill-sized steps (ops.moe)
 #   x += c y; h = LN_1 of the next layer (or the final norm's weight after the last layer)
@@ -460,8 +461,9 @@ class FanopelLayerW:
 
 class FanopelWeights:
     """Inference weights of a FanopelForCausalLM: q | k | gate stacked into one GEMM, the experts'
-    up projections stacked row-wise and their down projections side by side, norm weights, the
-    router, its correction and the distance-bias slopes in fp32."""
+    up projections stacked row-wise and their down projections side by side; norm weights, the
+    router's correction and the distance-bias slopes in fp32 (the router's weight stays in the
+    model dtype: its logits are formed in fp32 from the exact products, ``ops.moe.router_logits``)."""
 
     def __init__(self, model, tp_rank: int = 0, tp_size: int = 1):
         if tp_size != 1:
@@ -509,7 +511,7 @@ class FanopelWeights:
                                 rank_top=GROUP_RANK_TOP, norm=f32(p + "norm2"),
                                 up=torch.cat([t(y + f"e{e}.up") for e in range(E)], 0).contiguous(),
                                 down=torch.cat([t(y + f"e{e}.down") for e in range(E)], 1).contiguous(),
-                                router=f32(y + "router"), correction=f32(y + "correction"))
+                                router=t(y + "router").detach(), correction=f32(y + "correction"))
                 self.layers.append(L)
 
     def new_state(self, slots: int, num_blocks: int, block_size: int, device):
@@ -568,7 +570,7 @@ def run_fanopel_layers(w: FanopelWeights, st: FanopelState, tokens: torch.Tensor
         else:
             x, h2 = scaled_residual_layer_norm(x, y, c, f["norm"], eps, dt)
             # the router in fp32, on the (possibly 16-bit rounded) normed row
-            r = route_groups(h2.float() @ f["router"].t(), f["correction"], f["top"], f["groups"],
+            r = route_groups(router_logits(h2, f["router"]), f["correction"], f["top"], f["groups"],
                              f["keep"], f["scale"], f["sum_eps"], f["rank_top"])
             y2 = moe(h2, r, f["up"], f["down"], f["E"], f["top"], f["ff"], 0, "relu2", gated=False)
             x, h = scaled_residual_layer_norm(x, y2, c, nxt, eps, dt)

@@ -414,3 +414,14 @@ def test_experts_dense_and_grouped_match_oracle(device, dtype, E, top, n, keep, 
         got = fn(h, r, up, down, E, ff, 0, "relu2", gated=False)
         assert got.dtype == dtype
         close(got, want, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_router_logits_are_fp32_sums_of_exact_products(device, dtype):
+    from lumen.ops.moe import router_logits
+
+    h = rnd(300, 136, seed=90, dtype=dtype, device=device, scale=2.0)
+    w = rnd(12, 136, seed=91, dtype=dtype, device=device)
+    z = router_logits(h, w)
+    assert z.dtype == torch.float32
+    close(z, h.cpu().to(F64) @ w.cpu().to(F64).T, torch.float32)   # fp32 accuracy in every dtype
