@@ -799,9 +799,17 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
     bias).  ``window`` > 0: a row at position p only sees the keys j with p - j < window and,
     besides them, the sequence's first ``keep_first`` keys (at their true distances); tiles of
     keys between the two ranges are never loaded.  ``gate`` [T, H] (a view, any row stride):
-    head h's output is multiplied by sigmoid(gate[t, h]).  ``vt`` [blocks, Dv, block]: a per-block transposed copy of the
-    values (``latent_write`` keeps one); with it, one key/value head, values that are a prefix of
-    the key rows and a 16-bit dtype, the whole kernel runs on the matrix cores."""
+    head h's output is multiplied by sigmoid(gate[t, h]).  ``vt`` [blocks, Dv, block]: a per-block
+    transposed copy of the values (``latent_write`` keeps one); with it, one key/value head,
+    values that are a prefix of the key rows and a 16-bit dtype, the whole kernel runs on the
+    matrix cores.
+
+    Three kernels serve it.  The prompt portions of a step (``seg.q_tiles``) go to the tiled
+    matrix-core kernel of ``csrc/seqmix/window_attention.hip`` when the keys and values have caches
+    of their own, one query part, a head size it is built for, a 16-bit dtype and none of
+    temperature, logarithmic bias, head mixing or sink; the latent layout with ``vt`` goes to the
+    latent kernel; every other row (decoded rows, fp32, other shapes) to the row kernel.  A row's
+    result does not depend on which of them computed it beyond rounding."""
     from ._seqmix import DT, call, latent_attn_ok, use_seqmix, win_tiles_ok
 
     T, _, D1 = q1.shape

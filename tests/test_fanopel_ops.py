@@ -16,7 +16,8 @@ from test_dalavik_ops import CASES, F64, close, paged, rnd, segments
 
 from lumen.ops.attention import row_attention, row_norm_write
 from lumen.ops.embedding import embed_positions
-from lumen.ops.moe import moe_dense, moe_grouped, route_groups, scaled_act
+from lumen.ops.moe import (grouped_mm_ok, moe_dense, moe_grouped, moe_grouped_mm, route_groups,
+                           scaled_act)
 from lumen.ops.norm import scaled_residual_layer_norm, weight_layer_norm
 
 
@@ -414,6 +415,10 @@ def test_experts_dense_and_grouped_match_oracle(device, dtype, E, top, n, keep, 
         got = fn(h, r, up, down, E, ff, 0, "relu2", gated=False)
         assert got.dtype == dtype
         close(got, want, dtype)
+    if grouped_mm_ok(h, ff):                               # 16 bits on the GPU: no host in the loop
+        got = moe_grouped_mm(h, r, up, down, E, top, ff, 0, "relu2", gated=False)
+        assert got.dtype == dtype
+        close(got, want, dtype)
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
@@ -425,3 +430,34 @@ def test_router_logits_are_fp32_sums_of_exact_products(device, dtype):
     z = router_logits(h, w)
     assert z.dtype == torch.float32
     close(z, h.cpu().to(F64) @ w.cpu().to(F64).T, torch.float32)   # fp32 accuracy in every dtype
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("E,top,n,keep,ff,W,T", [(40, 2, 1, 1, 16, 64, 1000), (64, 4, 8, 2, 8, 40, 1200),
+                                                 (33, 1, 1, 1, 24, 128, 1100)])
+def test_grouped_gemm_form_with_idle_experts(dtype, E, top, n, keep, ff, W, T):
+    """The sync-free grouped form as ``moe`` picks it for many experts and few chosen: a correction
+    of -10 keeps a third of the experts from ever being chosen, so their groups are empty; one
+    expert takes every row."""
+    from lumen.ops.moe import moe
+
+    device = "cuda"
+    h = rnd(T, W, seed=70, dtype=dtype, device=device)
+    w = {"m.router": rnd(E, W, seed=71, scale=0.5), "m.correction": rnd(E, seed=72, scale=0.2)}
+    w["m.correction"][::3] = -10.0
+    w["m.correction"][1] = 10.0
+    for e in range(E):
+        w[f"m.e{e}.up"] = rnd(ff, W, seed=100 + e, dtype=dtype, scale=W ** -0.5)
+        w[f"m.e{e}.down"] = rnd(W, ff, seed=200 + e, dtype=dtype, scale=ff ** -0.5)
+    f = {"kind": "moe", "expert": {"ff": ff},
+         "router": {"experts": E, "top": top, "scale": 1.3, "groups": {"count": n, "keep": keep}}}
+    want = ref.moe_ff(h.cpu().to(F64), {k: v.to(F64) for k, v in w.items()}, "m.", f)
+    up = torch.cat([w[f"m.e{e}.up"] for e in range(E)], 0).to(device)
+    down = torch.cat([w[f"m.e{e}.down"] for e in range(E)], 1).to(device)
+    r = route_groups(h.float() @ w["m.router"].to(device).t(), w["m.correction"].to(device), top, n,
+                     keep, 1.3)
+    assert int((r[:, ::3] > 0).sum()) == 0 and bool((r[:, 1] > 0).all())
+    assert grouped_mm_ok(h, ff) and T * (E - 3 * top) >= 32768     # moe() takes the grouped GEMM
+    close(moe(h, r, up, down, E, top, ff, 0, "relu2", gated=False), want, dtype)
+    close(moe_grouped_mm(h, r, up, down, E, top, ff, 0, "relu2", gated=False), want, dtype)
