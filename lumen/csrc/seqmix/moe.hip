@@ -4,8 +4,9 @@
 //                  the row's `top` largest logits at their places, zero elsewhere).  One wave per
 //                  row: each lane keeps E / 64 logits in registers, `top` rounds of a wave-wide
 //                  arg-max (ties: lowest index).
-//   sm_route_groups  sigmoid router with a choice correction and a limit to the best groups of
-//                  experts: s = sigmoid(z), the choice ranks c = s + correction, a group of
+//   sm_route_groups  router with a choice correction and a limit to the best groups of
+//                  experts: s = sigmoid(z) (or the softmax of z over all experts; weights then
+//                  optionally un-normalised), the choice ranks c = s + correction, a group of
 //                  neighbouring experts ranks by the sum of its largest c, only experts of the
 //                  `keep` best groups are eligible, the `top` eligible experts with the largest c
 //                  get s / (sum of the chosen s + eps) * scale.  One wave per row, the row's c in
@@ -48,7 +49,7 @@ constexpr int kNone = 0x7fffffff;
 __global__ void __launch_bounds__(256)
 route_groups_kernel(const float* __restrict__ z, const float* __restrict__ corr,
                     float* __restrict__ out, int T, int E, int top, int n_groups, int keep,
-                    int rank_top, float scale, float sum_eps) {
+                    int rank_top, float scale, float sum_eps, int softmax, int normalize) {
   extern __shared__ float s_all[];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int row = blockIdx.x * 4 + wv;
@@ -57,8 +58,21 @@ route_groups_kernel(const float* __restrict__ z, const float* __restrict__ corr,
   float* rank = c + E;
   const float* zr = z + (long long)row * E;
   float* orow = out + (long long)row * E;
+  // the scores: sigmoids, or the softmax over all experts (maximum and sum wave-wide, fp32)
+  float smax = 0.f, sinv = 1.f;
+  if (softmax) {
+    smax = -INFINITY;
+    for (int e = lane; e < E; e += 64) smax = fmaxf(smax, zr[e]);
+    smax = wave_max(smax);
+    float ssum = 0.f;
+    for (int e = lane; e < E; e += 64) ssum += expf(zr[e] - smax);
+    sinv = 1.f / wave_sum(ssum);
+  }
+  const auto score = [&](int e) {
+    return softmax ? expf(zr[e] - smax) * sinv : sigmoid_f(zr[e]);
+  };
   for (int e = lane; e < E; e += 64) {
-    c[e] = sigmoid_f(zr[e]) + corr[e];
+    c[e] = score(e) + (corr != nullptr ? corr[e] : 0.f);
     orow[e] = 0.f;
   }
   __builtin_amdgcn_wave_barrier();
@@ -110,7 +124,7 @@ route_groups_kernel(const float* __restrict__ z, const float* __restrict__ corr,
       if (c[e] > bv) { bv = c[e]; bi = e; }          // ascending e: ties keep the lowest index
     wave_argmax(bv, bi);
     if (bi == kNone) break;                          // fewer than `top` eligible experts
-    den += sigmoid_f(zr[bi]);
+    den += score(bi);
     if ((bi & 63) == lane) {
       c[bi] = -INFINITY;
       if (n_mine < 16) mine[n_mine++] = bi;
@@ -118,8 +132,8 @@ route_groups_kernel(const float* __restrict__ z, const float* __restrict__ corr,
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   }
-  const float k = scale / (den + sum_eps);
-  for (int q = 0; q < n_mine; ++q) orow[mine[q]] = sigmoid_f(zr[mine[q]]) * k;
+  const float k = normalize ? scale / (den + sum_eps) : scale;
+  for (int q = 0; q < n_mine; ++q) orow[mine[q]] = score(mine[q]) * k;
 }
 
 template <typename T>
@@ -293,14 +307,14 @@ hipError_t sm_route_topk(const float* z, float* out, int T, int E, int top, hipS
 // z, out [T, E] fp32; corr [E] fp32.  4 * (E + n_groups) * 4 bytes of LDS per workgroup.
 hipError_t sm_route_groups(const float* z, const float* corr, float* out, int T, int E, int top,
                            int n_groups, int keep, int rank_top, float scale, float sum_eps,
-                           hipStream_t st) {
+                           int softmax, int normalize, hipStream_t st) {
   if (T == 0) return hipSuccess;
   if (E < 1 || E > 64 * kMaxPerLane || n_groups < 1 || E % n_groups || keep < 1 ||
       keep > n_groups || top < 1 || top > keep * (E / n_groups) || rank_top < 1 || rank_top > 4)
     return hipErrorInvalidValue;
   const size_t lds = 4 * (size_t)(E + n_groups) * sizeof(float);
   route_groups_kernel<<<(T + 3) / 4, 256, lds, st>>>(z, corr, out, T, E, top, n_groups, keep,
-                                                     rank_top, scale, sum_eps);
+                                                     rank_top, scale, sum_eps, softmax, normalize);
   return hipGetLastError();
 }
 

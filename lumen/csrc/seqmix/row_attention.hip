@@ -18,6 +18,10 @@
 //        s_h(j) <- sum_h' talk[h, h'] s_h'(j)                     (talk given)
 //        o_h     = sum_{j seen} exp(s_h(j)) v_g(j) / (sum_{j seen} exp(s_h(j)) + exp(sink_h))
 //        o_h    <- o_h * sigmoid(gate[t, h])                      (gate given)
+//     With `sigb` there is no softmax: o_h = sum_{j seen} sigmoid(s_h(j) + sigb_h) v_g(j), the
+//     weights as they are (no maximum is tracked; the running sum stays 1 so that the epilogue
+//     and the merge of key splits divide by 1).  With `vdiv` > 1 the value head of key head g is
+//     g / vdiv: several score maps (key heads) over one set of values.
 //     with temp(p) = 1 + tcoef * log(floor((p + 1) / tevery) + 1), g = h / (H / G), and the
 //     exp(sink_h) term only when a sink is given.  A row sees the keys j <= p; with a window > 0
 //     only those with p - j < window and, besides them, the first `keep` keys of the sequence: the
@@ -295,6 +299,7 @@ struct RowAttnArgs {
   const float *r1, *r2, *talk, *sink;
   const float* slopes; int window, keep;     // linear distance bias; window + kept first keys
   const T* gate; long long gater;            // per-head output gate logits [T][H], row stride
+  const float* sigb; int vdiv;               // sigmoid weights' per-head bias; key heads per value head
   int nsplit; float* ws_ml; float* ws_o;     // key splits: partial (max, sum) and accumulators
 };
 
@@ -379,6 +384,10 @@ row_attn_kernel(const RowAttnArgs<T> a) {
     const bool sk = a.sink != nullptr && hl < nh && blockIdx.z == 0;
     m[i] = sk ? a.sink[h0 + hl] : -INFINITY;     // the sink: a key of score sink_h, no value
     l[i] = sk ? 1.f : 0.f;
+    if (a.sigb != nullptr) {                     // un-normalised weights: (m, l) = (0, 1) once
+      m[i] = 0.f;
+      l[i] = blockIdx.z == 0 ? 1.f : 0.f;
+    }
     sreg[i] = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[i][e] = 0.f;
@@ -479,6 +488,10 @@ row_attn_kernel(const RowAttnArgs<T> a) {
         s = 0.f;
         for (int g = 0; g < nh; ++g) s += a.talk[h * a.H + h0 + g] * s_sc[(buf * a.HB + g) * 64 + lane];
       }
+      if (a.sigb != nullptr) {
+        s_p[hl * 64 + lane] = valid ? sigmoid_f(s + a.sigb[h]) : 0.f;
+        continue;
+      }
       s = valid ? s : -INFINITY;
       const float mn = fmaxf(m[i], wave_max(s));          // finite: a visited tile holds a seen key
       const float p = valid ? expf(s - mn) : 0.f;
@@ -496,7 +509,7 @@ row_attn_kernel(const RowAttnArgs<T> a) {
       // key/value head, four rows in flight before their products
       const int gw_lo = (h0 + hw0) / hpg, gw_hi = (h0 + min(nh, hw0 + HPW) - 1) / hpg;
       for (int g = gw_lo; g <= gw_hi; ++g) {
-        const T* vbase = a.vc + (long long)g * a.Dv;
+        const T* vbase = a.vc + (long long)(g / a.vdiv) * a.Dv;
         if (vvec) {
           if (grp < kpi) {
             constexpr int U = 4;
@@ -759,7 +772,8 @@ latent_attn_kernel(const RowAttnArgs<T> a, const T* __restrict__ vt) {
   // O[n][i] = O^T[channel (w NT + n) 16 + 4 kg + i][head hd]
   if (head_on) {
     if (a.nsplit == 1) {
-      const float inv = 1.f / l_run;
+      float inv = 1.f / l_run;
+      if (a.gate != nullptr) inv *= sigmoid_f(to_f32(a.gate[(long long)t * a.gater + h]));
       T* op = a.out + (long long)t * a.our + (long long)h * a.ouh;
 #pragma unroll
       for (int n = 0; n < NT; ++n) {
@@ -972,8 +986,8 @@ hipError_t sm_latent_attn(int dt, const void* q1, long long q1r, long long q1h, 
                           long long ouh, const int* tables, int maxb, const int* row_seg,
                           const int* positions, int T, int H, int bs, float scale, float softcap,
                           float tcoef, int tevery, const float* r1, const float* r2,
-                          const float* sink, int nsplit, float* ws_ml, float* ws_o,
-                          hipStream_t st) {
+                          const float* sink, const void* gate, long long gater, int nsplit,
+                          float* ws_ml, float* ws_o, hipStream_t st) {
   if (T == 0) return hipSuccess;
   const auto al = [](const void* p) { return (uintptr_t)p % 16 == 0; };
   if (!sm_latent_attn_ok(dt, Dv, D1 + D2, D1, bs) || nsplit < 1 || nsplit > 64 ||
@@ -986,13 +1000,13 @@ hipError_t sm_latent_attn(int dt, const void* q1, long long q1r, long long q1h, 
     RowAttnArgs<TT> a{(const TT*)q1, q1r, q1h, D1, (const TT*)q2, q2r, q2h, D2,               \
                       (const TT*)kc, krow, (const TT*)kc, krow, Dv, (TT*)out, our, ouh,       \
                       tables, maxb, row_seg, positions, H, 1, 16, bs, scale, softcap, tcoef,  \
-                      tevery, r1, r2, nullptr, sink, nullptr, 0, 0, nullptr, 0, nsplit,       \
-                      ws_ml, ws_o};                                                           \
+                      tevery, r1, r2, nullptr, sink, nullptr, 0, 0, (const TT*)gate, gater,   \
+                      nullptr, 1, nsplit, ws_ml, ws_o};                                       \
     hipError_t e = launch_latent_attn<TT>(a, (const TT*)vt, T, st);                           \
     if (e != hipSuccess) return e;                                                            \
     if (nsplit > 1)                                                                           \
       row_attn_combine_kernel<TT><<<dim3(T, H), 256, 0, st>>>(                                \
-          ws_ml, ws_o, (TT*)out, our, ouh, H, Dv, nsplit, (const TT*)nullptr, 0ll);           \
+          ws_ml, ws_o, (TT*)out, our, ouh, H, Dv, nsplit, (const TT*)gate, gater);            \
     return hipGetLastError();                                                                 \
   }
   SM_DISPATCH(dt, CALL)
@@ -1011,9 +1025,11 @@ hipError_t sm_row_attn(int dt, const void* q1, long long q1r, long long q1h, int
                        int bs, float scale, float softcap, float tcoef, int tevery,
                        const float* r1, const float* r2, const float* talk, const float* sink,
                        const float* slopes, int window, int keep, const void* gate,
-                       long long gater, int nsplit, float* ws_ml, float* ws_o, hipStream_t st) {
+                       long long gater, const float* sigb, int vdiv, int nsplit, float* ws_ml,
+                       float* ws_o, hipStream_t st) {
   if (T == 0) return hipSuccess;
   if (nsplit < 1 || nsplit > 64 || (nsplit > 1 && (!ws_ml || !ws_o))) return hipErrorInvalidValue;
+  if (vdiv < 1 || G % vdiv != 0 || (sigb && sink)) return hipErrorInvalidValue;
   if (H % G != 0 || HB < 1 || HB > 8 * kWaves || Dv > kMaxDv || (talk && HB < H) ||
       (D2 > 0 && q2 == nullptr) || window < 0 || keep < 0)
     return hipErrorInvalidValue;
@@ -1023,7 +1039,7 @@ hipError_t sm_row_attn(int dt, const void* q1, long long q1r, long long q1h, int
                       (const TT*)kc, krow, (const TT*)vc, vrow, Dv, (TT*)out, our, ouh,       \
                       tables, maxb, row_seg, positions, H, G, HB, bs, scale, softcap, tcoef,  \
                       tevery, r1, r2, talk, sink, slopes, window, keep, (const TT*)gate,      \
-                      gater, nsplit, ws_ml, ws_o};                                            \
+                      gater, sigb, vdiv, nsplit, ws_ml, ws_o};                                \
     return launch_row_attn<TT>(a, T, st);                                                     \
   }
   SM_DISPATCH(dt, CALL)

@@ -1,6 +1,7 @@
 """Model families: Llama / Llama-2 (7B, 13B, 70B-GQA), OPT (125m), Gedatar (hybrid stack),
-Dalavik (latent + grouped-query attention stack) and Fanopel (gated window attention + routed
-experts)."""
+Dalavik (latent + grouped-query attention stack), Fanopel (gated window attention + routed
+experts) and Foderax (parallel sigmoid-attention / minGRU, latent and differential attention
+layers with routed experts and depth-weighted layer inputs)."""
 from __future__ import annotations
 
 from typing import Optional
@@ -10,13 +11,15 @@ import torch
 from .config import PRESETS, ModelConfig, checkpoint_dir, get_config  # noqa: F401
 from .dalavik import DalavikForCausalLM  # noqa: F401
 from .fanopel import FanopelForCausalLM  # noqa: F401
+from .foderax import FoderaxForCausalLM  # noqa: F401
 from .gedatar import GedatarForCausalLM  # noqa: F401
 from .llama import LlamaForCausalLM  # noqa: F401
 from .opt import OPTForCausalLM  # noqa: F401
 
 
 MODEL_CLASSES = {"llama": LlamaForCausalLM, "opt": OPTForCausalLM, "gedatar": GedatarForCausalLM,
-                 "dalavik": DalavikForCausalLM, "fanopel": FanopelForCausalLM}
+                 "dalavik": DalavikForCausalLM, "fanopel": FanopelForCausalLM,
+                 "foderax": FoderaxForCausalLM}
 
 
 def build_model(name_or_cfg, dtype=torch.bfloat16, device=None, init: str = "auto",

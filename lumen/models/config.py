@@ -17,7 +17,7 @@ from typing import Optional
 
 @dataclass
 class ModelConfig:
-    arch: str = "llama"  # "llama" | "opt" | "gedatar" | "dalavik" | "fanopel"
+    arch: str = "llama"  # "llama" | "opt" | "gedatar" | "dalavik" | "fanopel" | "foderax"
     vocab_size: int = 32000
     hidden_size: int = 4096
     intermediate_size: int = 11008
@@ -50,12 +50,17 @@ class ModelConfig:
     # max_position_embeddings is the position table's row count): every sublayer's output is
     # multiplied by this before it joins the residual stream
     residual_mult: float = 1.0
+    # Foderax (layer_specs of "parallel" | "latent_attention" | "attention" mixers + routed
+    # experts, depth-weighted layer inputs): the embedding rows are multiplied by
+    # ``embedding_scale``; logits pass through cap * tanh(. / cap) when ``logit_softcap`` > 0
+    embedding_scale: float = 1.0
+    logit_softcap: float = 0.0
 
     @property
     def is_hybrid(self) -> bool:
         """Every layer names its own mixer and keeps its own kind of cache or state; such a stack
         is served by ``serve.hybrid_runner`` on the step's row segments."""
-        return self.arch in ("gedatar", "dalavik", "fanopel")
+        return self.arch in ("gedatar", "dalavik", "fanopel", "foderax")
 
     @property
     def head_dim(self) -> int:
@@ -77,6 +82,8 @@ class ModelConfig:
                 from .gedatar import tensor_shapes
             elif self.arch == "fanopel":
                 from .fanopel import tensor_shapes
+            elif self.arch == "foderax":
+                from .foderax import tensor_shapes
             else:
                 from .dalavik import tensor_shapes
 
@@ -201,7 +208,41 @@ def fanopel_to_dict(cfg: ModelConfig) -> dict:
             "eos_token_id": cfg.eos_token_id}
 
 
+def _foderax_to_config(d: dict) -> ModelConfig:
+    """config.json of a Foderax checkpoint: {"architecture": "Foderax", "vocab", "width",
+    "embedding": {"scale"}, "logit_softcap", "norm": {"eps"}, "layers": [{"type", "mixer",
+    "mlp"}, ...]}."""
+    layers = d["layers"]
+    if not layers:
+        raise ValueError("a Foderax config needs at least one layer")
+    for i, L in enumerate(layers):
+        if L.get("type") not in ("parallel", "latent_attention", "attention"):
+            raise ValueError(f"layer {i}: unknown mixer type {L.get('type')!r}")
+        kind = (L.get("mlp") or {}).get("kind", None)
+        if L.get("mlp") is not None and kind != "moe":
+            raise ValueError(f"layer {i}: unknown feed-forward kind {kind!r}")
+    return ModelConfig(
+        arch="foderax", vocab_size=int(d["vocab"]), hidden_size=int(d["width"]),
+        num_hidden_layers=len(layers), rms_norm_eps=float(d["norm"]["eps"]),
+        embedding_scale=float((d.get("embedding") or {}).get("scale", 1.0)),
+        logit_softcap=float(d.get("logit_softcap") or 0.0), layer_specs=layers,
+        intermediate_size=0, num_attention_heads=0, num_key_value_heads=0,
+        max_position_embeddings=1 << 20, tie_word_embeddings=True,
+        bos_token_id=int(d.get("bos_token_id", 0)), eos_token_id=int(d.get("eos_token_id", -1)),
+        pad_token_id=int(d.get("pad_token_id", 0)), name=d.get("_name_or_path", "foderax"))
+
+
+def foderax_to_dict(cfg: ModelConfig) -> dict:
+    """The checkpoint form of a Foderax configuration (inverse of ``_foderax_to_config``)."""
+    return {"architecture": "Foderax", "vocab": cfg.vocab_size, "width": cfg.hidden_size,
+            "embedding": {"scale": cfg.embedding_scale}, "logit_softcap": cfg.logit_softcap,
+            "norm": {"eps": cfg.rms_norm_eps}, "layers": cfg.layer_specs,
+            "eos_token_id": cfg.eos_token_id}
+
+
 def _hf_to_config(d: dict) -> ModelConfig:
+    if d.get("architecture") == "Foderax":
+        return _foderax_to_config(d)
     if d.get("architecture") == "Fanopel":
         return _fanopel_to_config(d)
     if d.get("architecture") == "Gedatar":
@@ -346,6 +387,34 @@ PRESETS = {
              "mlp": {"kind": "moe", "expert": {"ff": 56},
                      "router": {"experts": 5, "top": 2, "scale": 1.0,
                                 "groups": {"count": 1, "keep": 1}}}}]),
+    # parallel layer (sigmoid-weight attention beside a minGRU), latent attention with a sink and
+    # a per-head gate, differential attention (one layer borrowing the other's caches), softmax
+    # routed experts within the best groups, one layer without a feed-forward; depth-weighted
+    # layer inputs, scaled embedding, soft-capped logits
+    "tiny-foderax": dict(
+        arch="foderax", vocab_size=304, hidden_size=80, num_hidden_layers=4, rms_norm_eps=1e-5,
+        embedding_scale=8.0, logit_softcap=20.0, intermediate_size=0, num_attention_heads=0,
+        num_key_value_heads=0, max_position_embeddings=1 << 20, eos_token_id=-1,
+        tie_word_embeddings=True, name="tiny-foderax", layer_specs=[
+            {"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 24,
+                                            "scale": 0.25, "diff": 0.2,
+                                            "rot": {"base": 5000.0, "dims": 8}},
+             "mlp": {"kind": "moe", "expert": {"ff": 40},
+                     "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}}}},
+            {"type": "parallel", "mixer": {
+                "left": {"heads": 4, "kv_heads": 2, "dim": 24, "vdim": 16, "scale": 0.2,
+                         "rot": {"base": 20000.0, "dims": 16}},
+                "right": {"width": 72}, "left_scale": 0.7, "right_scale": 0.4},
+             "mlp": None},
+            {"type": "latent_attention", "mixer": {"heads": 3, "dim": 24, "vdim": 32,
+                                                   "kv_rank": 32, "q_rank": 40, "scale": 0.2},
+             "mlp": {"kind": "moe", "expert": {"ff": 48},
+                     "router": {"experts": 5, "top": 2, "groups": {"count": 1, "keep": 1}}}},
+            {"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 24,
+                                            "scale": 0.3, "diff": 0.35, "kv_from": 0,
+                                            "rot": {"base": 5000.0, "dims": 8}},
+             "mlp": {"kind": "moe", "expert": {"ff": 40},
+                     "router": {"experts": 6, "top": 3, "groups": {"count": 3, "keep": 2}}}}]),
     "tiny-opt": dict(arch="opt", vocab_size=512, hidden_size=64, intermediate_size=256,
                      ffn_dim=256, num_hidden_layers=2, num_attention_heads=4,
                      num_key_value_heads=4, max_position_embeddings=256, word_embed_proj_dim=64,

@@ -83,6 +83,10 @@ def load_hf_weights(model: nn.Module, path: str, strict: bool = True) -> None:
         from .fanopel import load_fanopel_weights
 
         return load_fanopel_weights(model, handles, path)
+    if model.config.arch == "foderax":
+        from .foderax import load_foderax_weights
+
+        return load_foderax_weights(model, handles, path)
     params = dict(model.named_parameters())
     for ours, srcs in _hf_name_map(model).items():
         if ours not in params:
@@ -112,13 +116,13 @@ def save_hf_weights(model: nn.Module, path: str, shard_bytes: int = 5 << 30) -> 
     os.makedirs(path, exist_ok=True)
     cfg = model.config
     if cfg.is_hybrid:
-        from .config import dalavik_to_dict, fanopel_to_dict, gedatar_to_dict
+        from .config import dalavik_to_dict, fanopel_to_dict, foderax_to_dict, gedatar_to_dict
 
         save_file({n: model.tensor(n).detach().cpu().contiguous() for n in model.tensor_names()},
                   os.path.join(path, "model.safetensors"), metadata={"format": "pt"})
         with open(os.path.join(path, "config.json"), "w") as f:
             to_dict = {"gedatar": gedatar_to_dict, "dalavik": dalavik_to_dict,
-                       "fanopel": fanopel_to_dict}[cfg.arch]
+                       "fanopel": fanopel_to_dict, "foderax": foderax_to_dict}[cfg.arch]
             json.dump(to_dict(cfg), f, indent=2)
         return
     params = dict(model.named_parameters())

@@ -38,14 +38,20 @@ SIGNATURES = {
     "sm_rotate_heads": "iplliiippi",
     "sm_latent_write": "iplppppppiiiiif",
     "sm_head_norm_write": "iplpppppiiiiif",
-    "sm_latent_attn": "i" "plli" "plli" "pl" "pi" "pll" "pi" "pp" "iii" "fffi" "ppp" "ipp",
+    "sm_latent_attn": "i" "plli" "plli" "pl" "pi" "pll" "pi" "pp" "iii" "fffi" "ppp" "pl" "ipp",
     "sm_row_attn": "i" "plli" "plli" "pl" "pli" "pll" "pi" "pp" "iiiii" "fffi" "pppp" "piipl"
-                   "ipp",
+                   "pi" "ipp",
     "sm_win_attn_tiles": "iplppppl" "pi" "pi" "pp" "iiii" "ff" "p" "iii",
     "sm_row_norm_write": "iplpppppiiif",
     "sm_layer_norm": "iippfppiif",
     "sm_embed_pos": "ipppppiiii",
-    "sm_route_groups": "pppiiiiiiff",
+    "sm_route_groups": "pppiiiiiiffii",
+    "sm_rotary_write": "iplppppiiiiipii",
+    "sm_min_gru": "iplpppppppiifppii",
+    "sm_diff_combine": "ipplpiiiifff",
+    "sm_depth_mix": "iipipppppppppppiif",
+    "sm_embed_scaled": "ipppiiif",
+    "sm_soft_cap": "ipplf",
     "sm_scaled_act": "ipppiiiii",
 }
 

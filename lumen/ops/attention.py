@@ -593,10 +593,11 @@ def latent_write_ref(z, w_norm, inv_freq, positions, slots, cache, R, dims, eps,
     c = zf[:, :R]
     c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * w_norm.float()
     kr = zf[:, R:].clone()
-    a = positions.float().view(-1, 1) * inv_freq.float().view(1, -1)
-    u, v = kr[:, 0:dims:2].clone(), kr[:, 1:dims:2].clone()
-    kr[:, 0:dims:2] = u * torch.cos(a) - v * torch.sin(a)
-    kr[:, 1:dims:2] = v * torch.cos(a) + u * torch.sin(a)
+    if dims:
+        a = positions.float().view(-1, 1) * inv_freq.float().view(1, -1)
+        u, v = kr[:, 0:dims:2].clone(), kr[:, 1:dims:2].clone()
+        kr[:, 0:dims:2] = u * torch.cos(a) - v * torch.sin(a)
+        kr[:, 1:dims:2] = v * torch.cos(a) + u * torch.sin(a)
     ok = slots >= 0
     cache.view(-1, cache.shape[-1])[slots[ok]] = torch.cat([c, kr], 1)[ok].to(cache.dtype)
     if vt is not None:
@@ -714,7 +715,7 @@ def row_norm_write(qk: torch.Tensor, wq: torch.Tensor, wk: torch.Tensor, slots: 
 
 def row_attention_ref(q1, q2, kcache, vcache, Dv, out, seg, H, G, scale, softcap=0.0,
                       q_temp=None, r1=None, r2=None, talk=None, sink=None, slopes=None,
-                      window=0, keep_first=0, gate=None):
+                      window=0, keep_first=0, gate=None, sigmoid_bias=None, v_div=1):
     T = q1.shape[0]
     D1 = q1.shape[2]
     D2 = q2.shape[2] if q2 is not None else 0
@@ -734,8 +735,9 @@ def row_attention_ref(q1, q2, kcache, vcache, Dv, out, seg, H, G, scale, softcap
         rows = tbl[js // bs] * bs + js % bs
         k = krows[rows][:, :G * Dk].float().view(-1, G, Dk)[:, hg]              # [n, H, Dk]
         v = vrows[rows].float()
-        v = (v[:, :G * Dv].view(-1, G, Dv) if G > 1 or vrows.shape[1] == Dv
-             else v[:, :Dv].view(-1, 1, Dv))[:, hg]                             # [n, H, Dv]
+        Gv = G // v_div
+        v = (v[:, :Gv * Dv].view(-1, Gv, Dv) if G > 1 or vrows.shape[1] == Dv
+             else v[:, :Dv].view(-1, 1, Dv))[:, hg // v_div]                    # [n, H, Dv]
         temp = 1.0
         if q_temp is not None and q_temp[0] != 0.0 and q_temp[1] > 0:
             temp = 1.0 + q_temp[0] * math.log((p + 1) // q_temp[1] + 1.0)
@@ -749,6 +751,12 @@ def row_attention_ref(q1, q2, kcache, vcache, Dv, out, seg, H, G, scale, softcap
             s = s - slopes.float().view(H, 1) * (p - js).float()
         if talk is not None:
             s = talk.float() @ s
+        if sigmoid_bias is not None:
+            o = torch.einsum("hn,nhd->hd", torch.sigmoid(s + sigmoid_bias.float().view(H, 1)), v)
+            if gate is not None:
+                o = o * torch.sigmoid(gate[t].float()).view(H, 1)
+            out[t] = o.to(out.dtype)
+            continue
         m = s.max(-1, keepdim=True).values
         if sink is not None:
             m = torch.maximum(m, sink.float().view(H, 1))
@@ -783,7 +791,8 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
                   vcache: torch.Tensor, Dv: int, out: torch.Tensor, seg, H: int, G: int,
                   scale: float, softcap: float = 0.0, q_temp=None, r1=None, r2=None, talk=None,
                   sink=None, vt: Optional[torch.Tensor] = None, slopes=None, window: int = 0,
-                  keep_first: int = 0, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  keep_first: int = 0, gate: Optional[torch.Tensor] = None,
+                  sigmoid_bias: Optional[torch.Tensor] = None, v_div: int = 1) -> torch.Tensor:
     """Causal attention of every row of a step against paged caches.
 
     q1 [T, H, D1] and (optionally) q2 [T, H, D2] are views with arbitrary row / head strides;
@@ -799,7 +808,11 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
     bias).  ``window`` > 0: a row at position p only sees the keys j with p - j < window and,
     besides them, the sequence's first ``keep_first`` keys (at their true distances); tiles of
     keys between the two ranges are never loaded.  ``gate`` [T, H] (a view, any row stride):
-    head h's output is multiplied by sigmoid(gate[t, h]).  ``vt`` [blocks, Dv, block]: a per-block
+    head h's output is multiplied by sigmoid(gate[t, h]).  ``sigmoid_bias`` [H]: no softmax -- a
+    seen key weighs sigmoid(s + sigmoid_bias_h), each weight on its own (nothing sums to one)
+    (a sink is meaningless then and refused).  ``v_div`` > 1: ``v_div`` consecutive key heads
+    share one value head (key head g reads value head g // v_div; ``vcache`` rows hold G / v_div
+    heads) -- several score maps over the same values.  ``vt`` [blocks, Dv, block]: a per-block
     transposed copy of the values (``latent_write`` keeps one); with it, one key/value head,
     values that are a prefix of the key rows and a 16-bit dtype, the whole kernel runs on the
     matrix cores.
@@ -817,17 +830,23 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
     Dk = D1 + D2
     if H % G:
         raise ValueError(f"{H} heads are not a multiple of {G} key/value heads")
+    v_div = int(v_div or 1)
+    if v_div < 1 or G % v_div:
+        raise ValueError(f"{G} key heads do not share values in groups of {v_div}")
+    if sigmoid_bias is not None and sink is not None:
+        raise ValueError("sigmoid weights are not normalised: a sink has no meaning")
     if not use_seqmix(q1):
         return row_attention_ref(q1, q2, kcache, vcache, Dv, out, seg, H, G, scale, softcap,
-                                 q_temp, r1, r2, talk, sink, slopes, window, keep_first, gate)
+                                 q_temp, r1, r2, talk, sink, slopes, window, keep_first, gate,
+                                 sigmoid_bias, v_div)
     if Dv > 512:
         raise ValueError(f"value size {Dv} > 512 is not supported")
     assert kcache.is_contiguous() and vcache.is_contiguous() and kcache.dtype == q1.dtype
     assert q1.stride(2) == 1 and out.stride(2) == 1 and (q2 is None or q2.stride(2) == 1)
     krow = kcache.shape[2:].numel()
     vrow = vcache.shape[2:].numel()
-    assert krow >= G * Dk and vrow >= G * Dv
-    for f in (r1, r2, talk, sink, slopes):
+    assert krow >= G * Dk and vrow >= (G // v_div) * Dv
+    for f in (r1, r2, talk, sink, slopes, sigmoid_bias):
         assert f is None or (f.dtype == torch.float32 and f.is_contiguous())
     window, keep_first = max(0, int(window or 0)), max(0, int(keep_first or 0))
     if gate is not None:
@@ -836,7 +855,8 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
     bs = kcache.shape[1]
     al8 = lambda x: x.data_ptr() % 16 == 0 and x.stride(0) % 8 == 0 and x.stride(1) % 8 == 0  # noqa: E731
     if (vt is not None and G == 1 and talk is None and vcache is kcache and D1 >= Dv
-            and slopes is None and window == 0 and gate is None
+            and slopes is None and window == 0 and sigmoid_bias is None
+            and (gate is None or gate.stride(1) == 1)
             and q1.dtype in (torch.bfloat16, torch.float16) and latent_attn_ok(DT[q1.dtype], Dv, Dk, D1, bs)
             and krow % 8 == 0 and al8(q1) and (q2 is None or al8(q2)) and out.data_ptr() % 8 == 0
             and out.stride(0) % 4 == 0 and out.stride(1) % 4 == 0):
@@ -852,7 +872,8 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
              q2, q2.stride(0) if q2 is not None else 0, q2.stride(1) if q2 is not None else 0, D2,
              kcache, krow, vt, Dv, out, out.stride(0), out.stride(1),
              seg.tables, seg.tables.shape[1], seg.row_seg, seg.positions, T, H, bs,
-             scale, float(softcap or 0.0), coef, every, r1, r2, sink, nsplit, ws_ml, ws_o)
+             scale, float(softcap or 0.0), coef, every, r1, r2, sink,
+             gate, gate.stride(0) if gate is not None else 0, nsplit, ws_ml, ws_o)
         return out
     # a step's prompt portions: tiles of consecutive rows of one segment on the matrix cores, when
     # nothing needs all heads of a (row, key) pair at once and the kernel has the head size; the
@@ -860,6 +881,7 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
     Tp = 0
     if (seg.q_tiles is not None and seg.tile_rows > 0 and q2 is None and talk is None
             and sink is None and r1 is None and q_temp is None and vcache is not kcache
+            and sigmoid_bias is None and v_div == 1
             and D1 == Dv and krow == G * D1 and vrow == G * Dv and win_tiles_ok(DT[q1.dtype], D1)
             and q1.stride(1) == D1 and q1.stride(0) % 8 == 0 and q1.data_ptr() % 16 == 0
             and out.stride(1) == Dv and out.stride(0) == H * Dv and out.data_ptr() % 8 == 0):
@@ -893,5 +915,42 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
          seg.tables, seg.tables.shape[1], row_seg, positions, T, H, G, HB,
          kcache.shape[1], scale, float(softcap or 0.0), coef, every, r1, r2, talk, sink,
          slopes, window, keep_first, gate, gate.stride(0) if gate is not None else 0,
-         nsplit, ws_ml, ws_o)
+         sigmoid_bias, v_div, nsplit, ws_ml, ws_o)
+    return out
+
+
+# ---- differential attention: two score maps per head combined, normed and gated -------------------
+# ``a`` holds both maps' outputs over the same values, laid out [T, G, 2, rep, Dv] (key head, map,
+# query head within the key head).  Head h = g * rep + r becomes
+#     o = a[g, 0, r] - lam * a[g, 1, r];   o <- o / sqrt(mean(o^2) + eps) * out_scale
+# and the concatenated heads are multiplied element-wise by sigmoid(gate).  fp32 throughout; only
+# the stored result is rounded.  (HIP: ``csrc/seqmix/foderax.hip``.)
+def diff_head_combine_ref(a, lam, out_scale, eps, gate, G, rep, Dv):
+    T = a.shape[0]
+    af = a.float().reshape(T, G, 2, rep, Dv)
+    o = af[:, :, 0] - lam * af[:, :, 1]                          # [T, G, rep, Dv]
+    o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * out_scale
+    o = o.reshape(T, G * rep * Dv)
+    if gate is not None:
+        o = o * torch.sigmoid(gate.float())
+    return o.to(a.dtype)
+
+
+def diff_head_combine(a: torch.Tensor, lam: float, out_scale: float, eps: float,
+                      gate: Optional[torch.Tensor], G: int, rep: int, Dv: int) -> torch.Tensor:
+    """a [T, G * 2 * rep * Dv] (contiguous) -> [T, G * rep * Dv] in a's dtype; ``gate``
+    [T, G * rep * Dv] (logits; a view with any row stride) or None."""
+    from ._seqmix import DT, call, use_seqmix
+
+    T = a.shape[0]
+    if a.shape[1:].numel() != G * 2 * rep * Dv:
+        raise ValueError(f"a has {a.shape[1:].numel()} columns, expected {G * 2 * rep * Dv}")
+    if not use_seqmix(a):
+        return diff_head_combine_ref(a, lam, out_scale, eps, gate, G, rep, Dv)
+    assert a.is_contiguous() and (gate is None or (gate.stride(1) == 1 and gate.dtype == a.dtype))
+    if Dv > 512:
+        raise ValueError(f"value size {Dv} > 512 is not supported")
+    out = torch.empty(T, G * rep * Dv, dtype=a.dtype, device=a.device)
+    call("sm_diff_combine", DT[a.dtype], a, gate, gate.stride(0) if gate is not None else 0, out,
+         T, G, rep, Dv, float(lam), float(out_scale), float(eps))
     return out

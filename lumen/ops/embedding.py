@@ -69,3 +69,41 @@ def embed_positions(tokens: torch.Tensor, positions: torch.Tensor, table: torch.
     call("sm_embed_pos", DT[table.dtype], table, pos_table, tokens, positions, out, T, W,
          table.shape[0], pos_table.shape[0])
     return out
+
+
+def embed_scaled_ref(tokens, table, scale, out):
+    out.copy_(table[tokens].float() * scale)
+    return out
+
+
+def embed_scaled(tokens: torch.Tensor, table: torch.Tensor, scale: float,
+                 out: torch.Tensor) -> torch.Tensor:
+    """table[token] * scale per row in fp32 into ``out`` [T, W] (fp32, contiguous): the start of a
+    residual stream whose embedding is multiplied by a constant.  (HIP
+    ``csrc/seqmix/foderax.hip``.)"""
+    from ._seqmix import DT, call, use_seqmix
+
+    if not use_seqmix(table):
+        return embed_scaled_ref(tokens, table, scale, out)
+    assert table.is_contiguous() and out.is_contiguous() and out.dtype == torch.float32
+    assert tokens.dtype == torch.int64 and tokens.is_contiguous()
+    T, W = tokens.shape[0], table.shape[1]
+    assert tuple(out.shape) == (T, W)
+    call("sm_embed_scaled", DT[table.dtype], table, tokens, out, T, W, table.shape[0], float(scale))
+    return out
+
+
+def soft_cap_ref(z, cap):
+    return cap * torch.tanh(z.float() / cap)
+
+
+def soft_cap(z: torch.Tensor, cap: float) -> torch.Tensor:
+    """cap * tanh(z / cap) element-wise in fp32 (z fp32 or 16-bit, contiguous) -> fp32."""
+    from ._seqmix import DT, call, use_seqmix
+
+    if not use_seqmix(z):
+        return soft_cap_ref(z, cap)
+    z = z.contiguous()
+    out = torch.empty(z.shape, dtype=torch.float32, device=z.device)
+    call("sm_soft_cap", DT[z.dtype], z, out, z.numel(), float(cap))
+    return out

@@ -58,10 +58,11 @@ def router_logits(h: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return h.float() @ w.float().t()
 
 
-def route_groups_ref(z, correction, top, n_groups, keep, scale, sum_eps=1e-20, rank_top=2):
+def route_groups_ref(z, correction, top, n_groups, keep, scale, sum_eps=1e-20, rank_top=2,
+                     score="sigmoid", normalize=True):
     T, E = z.shape
-    s = torch.sigmoid(z.float())
-    c = s + correction.float()
+    s = torch.softmax(z.float(), -1) if score == "softmax" else torch.sigmoid(z.float())
+    c = s + correction.float() if correction is not None else s
     if n_groups > 1 and keep < n_groups:
         per = E // n_groups
         cg = c.view(T, n_groups, per)
@@ -71,19 +72,22 @@ def route_groups_ref(z, correction, top, n_groups, keep, scale, sum_eps=1e-20, r
         c = cg.masked_fill(~allow.view(T, n_groups, 1), float("-inf")).reshape(T, E)
     idx = torch.sort(c, dim=-1, descending=True, stable=True).indices[:, :top]
     chosen = torch.gather(s, 1, idx)
-    wt = chosen / (chosen.sum(-1, keepdim=True) + sum_eps) * scale
+    wt = (chosen / (chosen.sum(-1, keepdim=True) + sum_eps) if normalize else chosen) * scale
     return torch.zeros_like(s).scatter_(1, idx, wt)
 
 
-def route_groups(z: torch.Tensor, correction: torch.Tensor, top: int, n_groups: int, keep: int,
-                 scale: float, sum_eps: float = 1e-20, rank_top: int = 2) -> torch.Tensor:
-    """Router logits z [T, E] (fp32) -> dense routing weights [T, E] (fp32) of a sigmoid router
-    with a choice correction and a limit to the best groups: the scores are s = sigmoid(z); the
-    choice ranks c = s + ``correction`` [E]; the experts form ``n_groups`` equal groups of
+def route_groups(z: torch.Tensor, correction: Optional[torch.Tensor], top: int, n_groups: int,
+                 keep: int, scale: float = 1.0, sum_eps: float = 1e-20, rank_top: int = 2,
+                 score: str = "sigmoid", normalize: bool = True) -> torch.Tensor:
+    """Router logits z [T, E] (fp32) -> dense routing weights [T, E] (fp32) of a router with a
+    choice correction and a limit to the best groups: the scores are s = sigmoid(z), or with
+    ``score`` = "softmax" the softmax of z over all experts; the
+    choice ranks c = s + ``correction`` [E] (None: c = s); the experts form ``n_groups`` equal groups of
     neighbours, a group ranks by the sum of its ``rank_top`` largest c, and only experts of the
     ``keep`` best groups can be chosen (``keep`` = ``n_groups``: no limit); the ``top`` eligible
     experts with the largest c get s_e / (sum of the chosen s + ``sum_eps``) * ``scale`` at their
-    places, all others zero.  Ties go to the lowest index."""
+    places (``normalize`` False: s_e * ``scale``, the scores as they are), all others zero.  Ties
+    go to the lowest index.  ``rank_top`` = 1 ranks a group by its best member."""
     from ._seqmix import call, use_seqmix
 
     T, E = z.shape
@@ -91,14 +95,18 @@ def route_groups(z: torch.Tensor, correction: torch.Tensor, top: int, n_groups: 
         raise ValueError(f"{E} experts do not form {n_groups} equal groups of which {keep} are kept")
     if not 1 <= top <= keep * (E // n_groups):
         raise ValueError(f"top {top} exceeds the {keep * (E // n_groups)} eligible experts")
+    if score not in ("sigmoid", "softmax"):
+        raise ValueError(f"unknown router score {score!r}")
     if not use_seqmix(z):
-        return route_groups_ref(z, correction, top, n_groups, keep, scale, sum_eps, rank_top)
+        return route_groups_ref(z, correction, top, n_groups, keep, scale, sum_eps, rank_top,
+                                score, normalize)
     assert z.dtype == torch.float32 and z.is_contiguous()
-    assert correction.dtype == torch.float32 and correction.is_contiguous()
+    assert correction is None or (correction.dtype == torch.float32 and correction.is_contiguous())
     if E > 1024:
         raise ValueError(f"route_groups supports at most 1024 experts, got {E}")
     out = torch.empty_like(z)
-    call("sm_route_groups", z, correction, out, T, E, top, n_groups, keep, rank_top, scale, sum_eps)
+    call("sm_route_groups", z, correction, out, T, E, top, n_groups, keep, rank_top, scale, sum_eps,
+         int(score == "softmax"), int(bool(normalize)))
     return out
 
 

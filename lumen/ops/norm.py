@@ -226,3 +226,55 @@ def scaled_residual_layer_norm(x: torch.Tensor, y: Optional[torch.Tensor], mult:
 def weight_layer_norm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype=None) -> torch.Tensor:
     """LN(x) * w of the fp32 rows ``x`` [T, W] in ``out_dtype``."""
     return scaled_residual_layer_norm(x, None, 0.0, w, eps, out_dtype or x.dtype)[1]
+
+
+# ---- depth-weighted layer inputs: layer scale, history, weighted average, next norm ---------------
+# A stack whose layer i reads a weighted average of everything before it keeps every layer's
+# result X_0 .. X_L of the step's rows in ``hist`` [L + 1, T, W] (fp32).  One pass per layer:
+#     X_n = x + sum_k scale_k * y_k          (the sublayers' outputs with per-channel scales)
+#     x  <- sum_{j <= n} mix[j] * X_j         (what the next layer reads)
+#     h   = x / sqrt(mean(x^2) + eps) * w     (its norm, in the compute dtype)
+# fp32 throughout; only h is rounded.  (HIP: ``csrc/seqmix/foderax.hip``.)
+def depth_mix_norm_ref(hist, n, x, ys, scales, mix, w, eps, out_dtype):
+    new = x.float().clone()
+    for y, sc in zip(ys, scales):
+        new += y.float() * sc.float()
+    hist[n] = new
+    xn = (hist[:n + 1] * mix.float().view(n + 1, 1, 1)).sum(0)
+    h = None
+    if w is not None:
+        h = (xn / torch.sqrt((xn * xn).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+    return xn, h
+
+
+def depth_mix_norm(hist: torch.Tensor, n: int, x: torch.Tensor, ys, scales, mix: torch.Tensor,
+                   w: Optional[torch.Tensor], eps: float, out_dtype=None):
+    """``hist`` [L + 1, T, W] fp32 holds X_0 .. X_(n-1); ``x`` [T, W] fp32 is the stream layer
+    n - 1 read; ``ys`` (up to three [T, W] sublayer outputs in the compute dtype) join it with the
+    per-channel fp32 ``scales`` [W] and the sum is stored as X_n; the new stream is
+    sum_j ``mix``[j] X_j over j = 0 .. n (``mix`` [n + 1] fp32) and, with ``w`` [W] (fp32, the
+    weight the normed row is multiplied by), h = rms_norm(stream) * w in ``out_dtype``.  Returns
+    (stream fp32 [T, W], h or None)."""
+    from ._seqmix import DT, call, use_seqmix
+
+    if not 1 <= len(ys) <= 3 or len(ys) != len(scales):
+        raise ValueError("one to three sublayer outputs, each with its scale")
+    if not 1 <= n < hist.shape[0] or mix.numel() != n + 1:
+        raise ValueError(f"history of {hist.shape[0]} entries, entry {n}, {mix.numel()} weights")
+    out_dtype = out_dtype or ys[0].dtype
+    if not use_seqmix(x):
+        return depth_mix_norm_ref(hist, n, x, ys, scales, mix, w, eps, out_dtype)
+    T, W = x.shape
+    assert hist.dtype == torch.float32 and hist.is_contiguous() and tuple(hist.shape[1:]) == (T, W)
+    assert x.dtype == torch.float32 and x.is_contiguous() and mix.dtype == torch.float32
+    for y, sc in zip(ys, scales):
+        assert y.is_contiguous() and y.shape == x.shape and y.dtype == ys[0].dtype
+        assert sc.dtype == torch.float32 and sc.is_contiguous() and sc.numel() == W
+    assert w is None or (w.dtype == torch.float32 and w.is_contiguous())
+    xn = torch.empty_like(x)
+    h = torch.empty(T, W, dtype=out_dtype, device=x.device) if w is not None else None
+    yp = list(ys) + [None] * (3 - len(ys))
+    sp = list(scales) + [None] * (3 - len(ys))
+    call("sm_depth_mix", DT[ys[0].dtype], DT[out_dtype], hist, n, x, yp[0], sp[0], yp[1], sp[1],
+         yp[2], sp[2], mix, w, xn, h, T, W, eps)
+    return xn, h

@@ -145,3 +145,62 @@ def delta_scan(r, k, v, wl, al, gl, w0, a_b, norm_w, state, seg: SegBatch, H: in
          _ld(gl), w0, a_b, norm_w, state, out, H * D, seg.cu, seg.slot, seg.start, seg.S, H, D,
          eps, decay_scale, key_eps)
     return out
+
+
+# ---- minGRU: an element-wise linear recurrence; gate and candidate depend on one token alone -------
+# Per channel, from S = 0 at a sequence's first token:
+#     z_t = sigmoid(zl_t + b_z);  u_t = xl_t + b_x;  c_t = u_t + shift (u_t >= 0) | sigmoid(u_t)
+#     S_t = (1 - z_t) S_(t-1) + z_t c_t;            out_t = S_t * silu(gl_t)
+# zl, xl, gl are column blocks of one fused projection's rows; gates, candidate and state are fp32
+# (``state`` [slots, width] carries S across steps); the result is stored in the compute dtype.
+def min_gru_scan_ref(zxg, b_z, b_x, state, seg: SegBatch, width, shift):
+    T = zxg.shape[0]
+    f = zxg.float()
+    z = torch.sigmoid(f[:, :width] + b_z.float())
+    u = f[:, width:2 * width] + b_x.float()
+    c = torch.where(u >= 0, u + shift, torch.sigmoid(u))
+    g = f[:, 2 * width:3 * width]
+    out = torch.empty(T, width, dtype=torch.float32, device=zxg.device)
+    cu, slots, starts = seg.cu.tolist(), seg.slot.tolist(), seg.start.tolist()
+    for s in range(seg.S):
+        a, b = cu[s], cu[s + 1]
+        if b == a:
+            continue
+        S = state[slots[s]].clone() if starts[s] > 0 else torch.zeros_like(state[slots[s]])
+        for t in range(a, b):
+            S = (1.0 - z[t]) * S + z[t] * c[t]
+            out[t] = S
+        state[slots[s]] = S
+    return (out * F.silu(g)).to(zxg.dtype)
+
+
+def min_gru_scan(zxg: torch.Tensor, b_z: torch.Tensor, b_x: torch.Tensor, state: torch.Tensor,
+                 seg: SegBatch, width: int, shift: float = 0.5) -> torch.Tensor:
+    """zxg [T, >= 3 * width] = [z logits | candidate pre-activations | output-gate logits] (a
+    fused projection's rows, unit column stride), biases [width] fp32 -> [T, width] in zxg's dtype,
+    ready for the output projection; ``state`` [slots, width] fp32 moves on by the step's rows (a
+    segment that starts at position 0 begins from zero whatever its slot holds)."""
+    from ._seqmix import DT, call, use_seqmix
+
+    if zxg.shape[1] < 3 * width:
+        raise ValueError(f"zxg has {zxg.shape[1]} columns, expected at least {3 * width}")
+    if not use_seqmix(zxg):
+        return min_gru_scan_ref(zxg, b_z, b_x, state, seg, width, shift)
+    assert zxg.stride(1) == 1 and state.dtype == torch.float32 and state.is_contiguous()
+    assert b_z.dtype == torch.float32 and b_x.dtype == torch.float32 and state.shape[1] == width
+    T = zxg.shape[0]
+    out = torch.empty(T, width, dtype=zxg.dtype, device=zxg.device)
+    # a step's prompt portions: every tile of rows reduced to its affine map S -> A S + B, then
+    # replayed from its true start state, so a long portion is not one serial walk; the decoded
+    # rows after them (one-row segments) and steps without tiles: one thread per channel
+    Tp = seg.tile_rows if seg.q_tiles is not None else 0
+    if Tp:
+        n = seg.q_tiles.shape[0]
+        ab = torch.empty(n * 2 * width, dtype=torch.float32, device=zxg.device)
+        call("sm_min_gru", DT[zxg.dtype], zxg, zxg.stride(0), b_z, b_x, state, out, seg.cu,
+             seg.slot, seg.start, 0, width, float(shift), ab, seg.q_tiles, n, seg.tile_size)
+    if T > Tp:
+        P = seg.S - (T - Tp) if Tp else 0              # decode rows are one-row segments
+        call("sm_min_gru", DT[zxg.dtype], zxg, zxg.stride(0), b_z, b_x, state, out, seg.cu[P:],
+             seg.slot[P:], seg.start[P:], seg.S - P, width, float(shift), None, None, 0, 0)
+    return out

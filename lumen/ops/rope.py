@@ -202,3 +202,63 @@ def rotate_interleaved_(x: torch.Tensor, positions: torch.Tensor, heads: int, he
     call("sm_rotate_heads", DT[x.dtype], x, x.stride(0), head_stride, heads, off, dims, inv_freq,
          positions, x.shape[0])
     return x
+
+
+# ---- rotary on the heads of a fused projection, keys and values into their paged caches ----------
+# One pass over a row of z = [q heads | k heads | values]: every q and k head of size D turns on
+# its first ``dims`` entries by the angle position * inv_freq[i] -- pairs (2i, 2i + 1) in the pair
+# layout, (i, i + dims / 2) in the half layout --, q in place, the turned k (also kept in z) and
+# the values as projected go to the cache rows ``slots``.  Angles and rotation are fp32.
+def rotary_write_ref(z, positions, slots, kcache, vcache, nq, nk, D, dims, inv_freq, half):
+    T = z.shape[0]
+    n = nq + nk
+    heads = z[:, :n * D].reshape(T, n, D).to(torch.float32, copy=True)
+    if dims:
+        a = positions.float().view(T, 1, 1) * inv_freq.float().view(1, 1, -1)
+        cs, sn = torch.cos(a), torch.sin(a)
+        if half:
+            u0, u1 = heads[..., :dims // 2].clone(), heads[..., dims // 2:dims].clone()
+            heads[..., :dims // 2] = u0 * cs - u1 * sn
+            heads[..., dims // 2:dims] = u1 * cs + u0 * sn
+        else:
+            u0, u1 = heads[..., 0:dims:2].clone(), heads[..., 1:dims:2].clone()
+            heads[..., 0:dims:2] = u0 * cs - u1 * sn
+            heads[..., 1:dims:2] = u1 * cs + u0 * sn
+    z[:, :n * D] = heads.reshape(T, n * D).to(z.dtype)
+    if kcache is not None:
+        ok = slots >= 0
+        kcache.view(-1, nk * D)[slots[ok]] = z[:, nq * D:n * D][ok].to(kcache.dtype)
+        vw = vcache.shape[2:].numel()
+        vcache.view(-1, vw)[slots[ok]] = z[:, n * D:n * D + vw][ok].to(vcache.dtype)
+
+
+def rotary_write(z: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor,
+                 kcache: Optional[torch.Tensor], vcache: Optional[torch.Tensor], nq: int, nk: int,
+                 D: int, dims: int, inv_freq: torch.Tensor, half: bool) -> None:
+    """z [T, >= (nq + nk) * D + value columns] (a fused projection's output; further columns are
+    left alone): the nq query heads and nk key heads (size D each, back to back from column 0)
+    are rotated in place on their first ``dims`` entries, ``half`` choosing the half layout over
+    the pair layout; the rotated keys go to ``kcache`` [blocks, block, ...] (rows of nk * D) and
+    the columns after the keys to ``vcache`` (rows of its own width) at ``slots`` (int64; -1
+    skips).  ``kcache`` None (nk must be 0): a layer that reads another's caches turns its queries
+    only."""
+    from ._seqmix import DT, call, use_seqmix
+
+    if dims % 2 or dims > D:
+        raise ValueError(f"rotary dims {dims} must be even and at most the head size {D}")
+    vw = vcache.shape[2:].numel() if vcache is not None else 0
+    if kcache is None and nk:
+        raise ValueError("key heads without a key cache")
+    if z.shape[1] < (nq + nk) * D + vw:
+        raise ValueError(f"z has {z.shape[1]} columns, expected at least {(nq + nk) * D + vw}")
+    if kcache is not None and kcache.shape[2:].numel() != nk * D:
+        raise ValueError(f"cache rows of {kcache.shape[2:].numel()} do not hold keys of {nk * D}")
+    if not use_seqmix(z):
+        return rotary_write_ref(z, positions, slots, kcache, vcache, nq, nk, D, dims, inv_freq,
+                                half)
+    assert z.stride(1) == 1 and positions.dtype == torch.int32
+    assert kcache is None or (kcache.is_contiguous() and vcache.is_contiguous()
+                              and kcache.dtype == z.dtype and vcache.dtype == z.dtype)
+    assert inv_freq.dtype == torch.float32 and inv_freq.numel() >= dims // 2
+    call("sm_rotary_write", DT[z.dtype], z, z.stride(0), positions, slots, kcache, vcache,
+         z.shape[0], nq, nk, D, dims, inv_freq, int(bool(half)), vw)

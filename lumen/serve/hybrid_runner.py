@@ -1,11 +1,11 @@
 """Serving runner for stacks whose layers each name their own mixer (Gedatar, Dalavik,
-Fanopel): paged caches + per-sequence recurrent state.
+Fanopel, Foderax): paged caches + per-sequence recurrent state.
 
-Three families share the runner, the segments, the block manager and the hipGraph decode; each
+Four families share the runner, the segments, the block manager and the hipGraph decode; each
 has its weights class (stacked projections, fp32 constants), its caches and its step function:
 Gedatar (``HybridWeights`` / ``HybridState`` / ``run_layers``, described next), Dalavik
-(``DalavikWeights`` / ``DalavikState``) and Fanopel (``FanopelWeights`` / ``FanopelState``),
-further down.
+(``DalavikWeights`` / ``DalavikState``), Fanopel (``FanopelWeights`` / ``FanopelState``) and
+Foderax (``FoderaxWeights`` / ``FoderaxState``), further down.
 
 One step function for prefill chunks, decode rows and mixtures of both.  The rows of a step are
 cut into segments (``ops.segments.SegBatch``: one per chunk, one per decode row); per layer
@@ -41,15 +41,16 @@ import torch.nn.functional as F
 
 from ..models.config import ModelConfig
 from ..models.gedatar import DELTA_DECAY, DELTA_KEY_EPS
-from ..ops.attention import (chunk_sink_attention, head_norm_write, latent_write, row_attention,
-                             row_norm_write, transposed_values_ok, write_key_cache)
+from ..ops.attention import (chunk_sink_attention, diff_head_combine, head_norm_write,
+                             latent_write, row_attention, row_norm_write, transposed_values_ok,
+                             write_key_cache)
 from ..ops.conv import dyt_canon
-from ..ops.embedding import embed_positions, gated_token_slice
+from ..ops.embedding import embed_positions, embed_scaled, gated_token_slice, soft_cap
 from ..ops.moe import gated_act, moe, route_groups, route_topk, router_logits
-from ..ops.norm import (dyt, dyt_residual, group_rms_norm, group_rms_residual,
+from ..ops.norm import (depth_mix_norm, dyt, dyt_residual, group_rms_norm, group_rms_residual,
                         scaled_residual_layer_norm, weight_layer_norm)
-from ..ops.recurrent import delta_scan, token_shift, wkv_scan
-from ..ops.rope import rotate_interleaved_
+from ..ops.recurrent import delta_scan, min_gru_scan, token_shift, wkv_scan
+from ..ops.rope import rotary_write, rotate_interleaved_
 from ..ops.segments import SegBatch, whole_sequences
 from .model_runner import ModelRunner, StepInput
 
@@ -167,6 +168,17 @@ def key_bytes_per_token(cfg: ModelConfig, dtype_bytes: int = 2) -> int:
     if cfg.arch == "fanopel":                  # normed keys + the keys as projected (the values)
         return max(1, sum(2 * L["mixer"]["kv_heads"] * L["mixer"]["dim"]
                           for L in cfg.layer_specs) * dtype_bytes)
+    if cfg.arch == "foderax":
+        n = 0
+        for L in cfg.layer_specs:
+            m = L["mixer"]
+            if L["type"] == "parallel":
+                n += m["left"]["kv_heads"] * (m["left"]["dim"] + m["left"]["vdim"])
+            elif L["type"] == "latent_attention":
+                n += 2 * m["kv_rank"]                      # the latent twice: rows and transposed
+            elif m.get("kv_from") is None:
+                n += m["kv_heads"] * (2 * m["dim"] + m["vdim"])
+        return max(1, n * dtype_bytes)
     if cfg.arch == "dalavik":
         n = 0
         for L in cfg.layer_specs:
@@ -183,6 +195,9 @@ def key_bytes_per_token(cfg: ModelConfig, dtype_bytes: int = 2) -> int:
 def state_bytes_per_slot(cfg: ModelConfig) -> int:
     if cfg.arch in ("dalavik", "fanopel"):
         return 0
+    if cfg.arch == "foderax":
+        return 4 * sum(L["mixer"]["right"]["width"] for L in cfg.layer_specs
+                       if L["type"] == "parallel")
     n = 0
     for L in cfg.layer_specs:
         n += max(cfg.canon_taps - 1, 0) * cfg.hidden_size
@@ -579,7 +594,271 @@ def run_fanopel_layers(w: FanopelWeights, st: FanopelState, tokens: torch.Tensor
     return x
 
 
-WEIGHTS = {"gedatar": HybridWeights, "dalavik": DalavikWeights, "fanopel": FanopelWeights}
+# ---- Foderax: parallel layers on depth-weighted inputs ---------------------------------------------
+#
+#   hist[0] = embed[token] * scale (fp32);  x = hist[0];  h = rms(x) * (1 + w)   (model dtype)
+#   per layer i, every sublayer reading the same h:
+#   parallel
+#       z  = [W_q ; W_k ; W_v ; W_z ; W_x ; W_g] h     one GEMM (left attention | right recurrence)
+#       q, k turned in the half layout, k and v into their caches                 (rotary_write)
+#       o  = row_attention(sigmoid weights: sigmoid(score + pb_h), not normalised);  y_l = W_ol o
+#       r  = min_gru_scan(z's last three blocks, the slot's fp32 state);          y_r = W_or r
+#   latent_attention
+#       z  = [W_dq ; W_dkv ; W_g] h                    one GEMM
+#       cache row <- rms(z_kv) * w                      (latent_write, + the per-block transpose)
+#       q  = W_uq (rms(z_q) * w);  qa = per-head W_uk^T q   (the query in the latent space)
+#       ol = row_attention(qa against the cached rows, value = the row, sink, per-head gate)
+#       y  = W_o (per-head W_uv ol)
+#   attention (differential)
+#       z  = [W_q' ; W_k ; W_v ; W_g] h + b            one GEMM; q' = q's rows reordered to
+#            [key head][map][query head of the group], so that the two maps are 2 H heads on 2 G
+#            key heads sharing G value heads
+#       q', k turned in the pair layout, k and v into their caches (a borrowing layer: q' only)
+#       a  = row_attention(2 H heads, v_div = 2);  o = diff_head_combine(a, lambda, 1 - diff, gate)
+#       y  = W_o o
+#   experts: r = route_groups(softmax scores, groups ranked by their best member, weights as they
+#            are);  y_f = [W_down_e] (relu(W_up h)^2 * r)
+#   hist[i + 1] = x + ls1 * y (+ ls2 * y_f);  x = sum_j dwa[j] hist[j];  h = rms(x) * (1 + w_next)
+#                                                                          (depth_mix_norm, one pass)
+#   logits = cap * tanh((embed h_final) / cap)         fp32 product of the 16-bit operands
+#
+# fp32: the stream and its history, norms, angles, scores, sigmoid / softmax weights, sinks, the
+# map combination and its norm, gates' sigmoids, the recurrence (gates, candidate, state), the
+# router; model dtype: GEMMs and what they store.
+@dataclass
+class FoderaxLayerW:
+    kind: str                       # parallel | latent_attention | attention
+    m: dict                         # the mixer's sizes and constants
+    norm1: torch.Tensor             # 1 + the stored offset, fp32
+    w: Dict[str, torch.Tensor] = field(default_factory=dict)
+    c: dict = field(default_factory=dict)      # host constants
+    ff: Optional[dict] = None
+    kv_layer: int = -1              # attention: the layer whose caches it reads
+
+
+def _pad_rows(parts, dtype, dev):
+    """Stack projection weights row-wise, zero rows added up to a multiple of 8 output columns (so
+    that every view of the GEMM's output keeps 16-byte row strides)."""
+    rows = sum(p.shape[0] for p in parts)
+    pad = -rows % 8
+    if pad:
+        parts = list(parts) + [torch.zeros(pad, parts[0].shape[1], dtype=dtype, device=dev)]
+    return torch.cat(parts, 0).contiguous()
+
+
+class FoderaxWeights:
+    """Inference weights of a FoderaxForCausalLM: projections that share the layer's one normed
+    input are stacked into one GEMM, differential queries are reordered by key head and map, the
+    per-head up projections of latent attention are laid out for batched GEMMs, the experts' up
+    projections are stacked row-wise and their down projections side by side; norm weights (with
+    the 1 added), layer scales (with the mixers' constant scales folded in), depth weights and
+    per-head constants are fp32."""
+
+    def __init__(self, model, tp_rank: int = 0, tp_size: int = 1):
+        if tp_size != 1:
+            raise NotImplementedError("Foderax models are served at tensor-parallel size 1")
+        from ..models.foderax import CANDIDATE_SHIFT, router_groups
+        from ..ops.rope import interleaved_inv_freq
+
+        cfg: ModelConfig = model.config
+        self.cfg = cfg
+        t = model.tensor
+        f32 = lambda n: t(n).detach().float().contiguous()  # noqa: E731
+        f64 = lambda n: t(n).detach().double()  # noqa: E731
+        self.dtype = dt = t("embed").dtype
+        dev = t("embed").device
+        self.embed = t("embed").detach()
+        self.lm_head = self.embed                           # tied, unscaled
+        self.final = (1.0 + f32("final.norm")).contiguous()
+        self.vocab_shard = cfg.vocab_size
+        self.shift = float(CANDIDATE_SHIFT)
+        self.layers: List[FoderaxLayerW] = []
+        with torch.no_grad():
+            for i, spec in enumerate(cfg.layer_specs):
+                p, m = f"l{i}.", spec["mixer"]
+                x = p + "mix."
+                L = FoderaxLayerW(spec["type"], m, (1.0 + f32(p + "norm1")).contiguous())
+                ls1 = f32(p + "ls1")
+                if L.kind == "parallel":
+                    a = m["left"]
+                    lt, rt = x + "left.", x + "right."
+                    L.w["in"] = _pad_rows([t(lt + "q"), t(lt + "k"), t(lt + "v"), t(rt + "z"),
+                                           t(rt + "x"), t(rt + "g")], dt, dev)
+                    L.w["pb"] = f32(lt + "pb")
+                    L.w["b_z"], L.w["b_x"] = f32(rt + "z.b"), f32(rt + "x.b")
+                    L.w["o_l"], L.w["o_r"] = t(lt + "o").detach(), t(rt + "o").detach()
+                    L.w["inv_freq"] = interleaved_inv_freq(a["rot"]["dims"], a["rot"]["base"], dev)
+                    L.w["scales"] = [(ls1 * float(m["left_scale"])).contiguous(),
+                                     (ls1 * float(m["right_scale"])).contiguous()]
+                elif L.kind == "latent_attention":
+                    H, D, Dv, R = m["heads"], m["dim"], m["vdim"], m["kv_rank"]
+                    L.w["in"] = _pad_rows([t(x + "dq"), t(x + "dkv"), t(x + "g")], dt, dev)
+                    L.w["dq_norm"], L.w["dkv_norm"] = f32(x + "dq.norm"), f32(x + "dkv.norm")
+                    L.w["uq"] = t(x + "uq").detach()
+                    L.w["uk"] = t(x + "uk").detach().view(H, D, R)                   # q_h @ uk[h]
+                    L.w["uvT"] = t(x + "uv").detach().view(H, Dv, R).transpose(1, 2).contiguous()
+                    L.w["sink"] = f32(x + "sink")
+                    L.w["o"] = t(x + "o").detach()
+                    L.w["scales"] = [ls1]
+                else:
+                    H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+                    rep = H // G
+                    own = m.get("kv_from") is None
+                    L.kv_layer = i if own else int(m["kv_from"])
+                    # query rows [head][map][D] -> [key head][map][head of the group][D]
+                    perm = (torch.arange(2 * H * D, device=dev).view(G, rep, 2, D)
+                            .permute(0, 2, 1, 3).reshape(-1))
+                    parts = [t(x + "q").detach()[perm]]
+                    bias = [t(x + "q.b").detach()[perm]]
+                    if own:
+                        parts += [t(x + "k"), t(x + "v")]
+                        bias += [t(x + "k.b"), t(x + "v.b")]
+                    parts.append(t(x + "g"))
+                    bias.append(torch.zeros(H * Dv, dtype=dt, device=dev))
+                    L.w["in"] = _pad_rows(parts, dt, dev)
+                    b = torch.cat(bias, 0)
+                    L.w["in_b"] = torch.cat([b, b.new_zeros(L.w["in"].shape[0] - b.shape[0])])
+                    L.c["lam"] = float(torch.exp((f64(x + "lq1") * f64(x + "lk1")).sum())
+                                       - torch.exp((f64(x + "lq2") * f64(x + "lk2")).sum())
+                                       + float(m["diff"]))
+                    L.w["inv_freq"] = interleaved_inv_freq(m["rot"]["dims"], m["rot"]["base"], dev)
+                    L.w["o"] = t(x + "o").detach()
+                    L.w["scales"] = [ls1]
+                L.w["dwa"] = f32(p + "dwa")
+                f = spec.get("mlp")
+                if f:
+                    y = p + "mlp."
+                    r = f["router"]
+                    E = r["experts"]
+                    n, keep = router_groups(f)
+                    L.ff = dict(E=E, top=int(r["top"]), ff=int(f["expert"]["ff"]), groups=n, keep=keep,
+                                up=torch.cat([t(y + f"e{e}.up") for e in range(E)], 0).contiguous(),
+                                down=torch.cat([t(y + f"e{e}.down") for e in range(E)], 1).contiguous(),
+                                router=t(y + "router").detach(), ls2=f32(p + "ls2"))
+                self.layers.append(L)
+
+    def new_state(self, slots: int, num_blocks: int, block_size: int, device):
+        return FoderaxState(self, slots, num_blocks, block_size, device)
+
+    def run_layers(self, st, tokens, seg, observe=None) -> torch.Tensor:
+        return run_foderax_layers(self, st, tokens, seg, observe)
+
+    def head(self, x: torch.Tensor) -> torch.Tensor:
+        h = group_rms_norm(x, self.final, 1, self.cfg.rms_norm_eps, self.dtype)
+        z = router_logits(h, self.lm_head)       # fp32 logits from the 16-bit (or fp32) operands
+        cap = self.cfg.logit_softcap
+        return soft_cap(z, cap) if cap > 0 else z
+
+
+class FoderaxState:
+    """Caches and state of a Foderax model.  Paged through the engine's block manager: rotated keys
+    and values of every parallel layer's attention half, the normed latent of every
+    latent-attention layer (+ its per-block transpose where the matrix-core value product can use
+    it), both maps' rotated keys and the values of every differential layer that projects its own
+    (a borrowing layer reads the lender's).  Per state slot (+ one spare for graph padding rows):
+    the fp32 recurrent state [slots + 1, width] of every parallel layer's recurrence."""
+
+    def __init__(self, w: FoderaxWeights, slots: int, num_blocks: int, block_size: int, device):
+        self.slots = slots
+        self.spare = slots
+        kw = dict(dtype=w.dtype, device=device)
+        n = len(w.layers)
+        self.k: List[Optional[torch.Tensor]] = [None] * n
+        self.v: List[Optional[torch.Tensor]] = [None] * n
+        self.lat: List[Optional[torch.Tensor]] = [None] * n
+        self.latT: List[Optional[torch.Tensor]] = [None] * n
+        self.S: List[Optional[torch.Tensor]] = [None] * n
+        for i, L in enumerate(w.layers):
+            m = L.m
+            if L.kind == "parallel":
+                a = m["left"]
+                self.k[i] = torch.zeros(num_blocks, block_size, a["kv_heads"], a["dim"], **kw)
+                self.v[i] = torch.zeros(num_blocks, block_size, a["kv_heads"], a["vdim"], **kw)
+                self.S[i] = torch.zeros(slots + 1, m["right"]["width"], dtype=torch.float32,
+                                        device=device)
+            elif L.kind == "latent_attention":
+                R = m["kv_rank"]
+                self.lat[i] = torch.zeros(num_blocks, block_size, R, **kw)
+                if transposed_values_ok(w.dtype, R, 0, block_size, device):
+                    self.latT[i] = torch.zeros(num_blocks, R, block_size, **kw)
+            elif L.kv_layer == i:
+                self.k[i] = torch.zeros(num_blocks, block_size, 2 * m["kv_heads"], m["dim"], **kw)
+                self.v[i] = torch.zeros(num_blocks, block_size, m["kv_heads"], m["vdim"], **kw)
+
+
+def run_foderax_layers(w: FoderaxWeights, st: FoderaxState, tokens: torch.Tensor, seg: SegBatch,
+                       observe=None) -> torch.Tensor:
+    """The step function: token ids [T] + their segments -> the fp32 stream [T, W] the head
+    reads; caches and recurrent state in ``st`` move on by the step's rows."""
+    cfg = w.cfg
+    dt = w.dtype
+    eps = cfg.rms_norm_eps
+    T = tokens.shape[0]
+    dev = tokens.device
+    n_layers = len(w.layers)
+    hist = torch.empty(n_layers + 1, T, cfg.hidden_size, dtype=torch.float32, device=dev)
+    x = embed_scaled(tokens, w.embed, cfg.embedding_scale, hist[0])
+    h = group_rms_norm(x, w.layers[0].norm1, 1, eps, dt)
+    for i, L in enumerate(w.layers):
+        m = L.m
+        if L.kind == "parallel":
+            a = m["left"]
+            H, G, D, Dv, Wd = a["heads"], a["kv_heads"], a["dim"], a["vdim"], m["right"]["width"]
+            z = F.linear(h, L.w["in"])
+            rotary_write(z, seg.positions, seg.cache_slots, st.k[i], st.v[i], H, G, D,
+                         int(a["rot"]["dims"]), L.w["inv_freq"], True)
+            o = torch.empty(T, H, Dv, dtype=dt, device=dev)
+            row_attention(z[:, :H * D].view(T, H, D), None, st.k[i], st.v[i], Dv, o, seg, H, G,
+                          float(a["scale"]), sigmoid_bias=L.w["pb"])
+            c0 = (H + G) * D + G * Dv
+            r = min_gru_scan(z[:, c0:c0 + 3 * Wd], L.w["b_z"], L.w["b_x"], st.S[i], seg, Wd,
+                             w.shift)
+            ys = [F.linear(o.view(T, H * Dv), L.w["o_l"]), F.linear(r, L.w["o_r"])]
+        elif L.kind == "latent_attention":
+            H, D, Dv, R, Q = m["heads"], m["dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+            z = F.linear(h, L.w["in"])
+            latent_write(z[:, Q:Q + R], L.w["dkv_norm"], None, seg.positions, seg.cache_slots,
+                         st.lat[i], R, 0, eps, st.latT[i])
+            q = F.linear(group_rms_norm(z[:, :Q], L.w["dq_norm"], 1, eps, dt), L.w["uq"])
+            qa = torch.bmm(q.view(T, H, D).transpose(0, 1), L.w["uk"])          # [H, T, R]
+            ol = torch.empty(H, T, R, dtype=dt, device=dev)
+            row_attention(qa.transpose(0, 1), None, st.lat[i], st.lat[i], R, ol.transpose(0, 1),
+                          seg, H, 1, float(m["scale"]), sink=L.w["sink"], vt=st.latT[i],
+                          gate=z[:, Q + R:Q + R + H])
+            o = torch.empty(T, H, Dv, dtype=dt, device=dev)
+            torch.bmm(ol, L.w["uvT"], out=o.transpose(0, 1))
+            ys = [F.linear(o.view(T, H * Dv), L.w["o"])]
+        else:
+            H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            own = L.kv_layer == i
+            z = F.linear(h, L.w["in"], L.w["in_b"])
+            rotary_write(z, seg.positions, seg.cache_slots, st.k[i], st.v[i], 2 * H,
+                         2 * G if own else 0, D, int(m["rot"]["dims"]), L.w["inv_freq"], False)
+            av = torch.empty(T, 2 * H, Dv, dtype=dt, device=dev)
+            row_attention(z[:, :2 * H * D].view(T, 2 * H, D), None, st.k[L.kv_layer],
+                          st.v[L.kv_layer], Dv, av, seg, 2 * H, 2 * G, float(m["scale"]), v_div=2)
+            g0 = 2 * H * D + ((2 * G * D + G * Dv) if own else 0)
+            o = diff_head_combine(av.view(T, 2 * H * Dv), L.c["lam"], 1.0 - float(m["diff"]), eps,
+                                  z[:, g0:g0 + H * Dv], G, H // G, Dv)
+            ys = [F.linear(o, L.w["o"])]
+        scales = list(L.w["scales"])
+        f = L.ff
+        if f is not None:
+            # the router in fp32, on the (possibly 16-bit rounded) normed row
+            r = route_groups(router_logits(h, f["router"]), None, f["top"], f["groups"], f["keep"],
+                             1.0, rank_top=1, score="softmax", normalize=False)
+            ys.append(moe(h, r, f["up"], f["down"], f["E"], f["top"], f["ff"], 0, "relu2",
+                          gated=False))
+            scales.append(f["ls2"])
+        nxt = w.layers[i + 1].norm1 if i + 1 < n_layers else None
+        x, h = depth_mix_norm(hist, i + 1, x, ys, scales, L.w["dwa"], nxt, eps, dt)
+        if observe is not None:
+            observe(i, x)
+    return x
+
+
+WEIGHTS = {"gedatar": HybridWeights, "dalavik": DalavikWeights, "fanopel": FanopelWeights,
+           "foderax": FoderaxWeights}
 
 
 class HybridRunner(ModelRunner):
