@@ -400,7 +400,7 @@ PRESETS = {
                                             "scale": 0.25, "diff": 0.2,
                                             "rot": {"base": 5000.0, "dims": 8}},
              "mlp": {"kind": "moe", "expert": {"ff": 40},
-                     "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}}}},
+                     "router": {"experts": 8, "top": 3, "groups": {"count": 4, "keep": 2}}}},
             {"type": "parallel", "mixer": {
                 "left": {"heads": 4, "kv_heads": 2, "dim": 24, "vdim": 16, "scale": 0.2,
                          "rot": {"base": 20000.0, "dims": 16}},
