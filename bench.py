@@ -495,7 +495,7 @@ def main():
                          "per-layer-mixer design (--hybrid_family) beside Llama at equal size, "
                          "one GPU (lumen/bench/hybrid_bench.py)")
     ap.add_argument("--hybrid_family", default="gedatar",
-                    choices=["gedatar", "dalavik", "fanopel"])
+                    choices=["gedatar", "dalavik", "fanopel", "foderax"])
     ap.add_argument("--hybrid_widths", default="2048,4096")
     ap.add_argument("--hybrid_batch", default="8,64", help="sequences per step (comma list)")
     ap.add_argument("--hybrid_prompt", type=int, default=512)

@@ -1,9 +1,11 @@
-"""Prefill / decode throughput of a per-layer-mixer design (Gedatar, Dalavik, Fanopel) beside
-Llama at equal size.
+"""Prefill / decode throughput of a per-layer-mixer design (Gedatar, Dalavik, Fanopel, Foderax)
+beside Llama at equal size.
 
-``python bench.py --hybrid [--hybrid_family dalavik|fanopel]`` (one GPU).  Fanopel also runs
-beside the closest design the framework already had: a Gedatar stack of attention layers (keys
-as values) with routed experts of the same shapes.  Both models get random
+``python bench.py --hybrid [--hybrid_family dalavik|fanopel|foderax]`` (one GPU).  Fanopel also
+runs beside the closest design the framework already had: a Gedatar stack of attention layers
+(keys as values) with routed experts of the same shapes; Foderax beside Dalavik (latent and
+grouped-query attention through the same row kernels) and Fanopel (experts of the same shapes).
+All models get random
 weights of layer shapes that resemble real models (width 2048 / 4096, head size 128 / 64, FFN 2.75 x width, vocab 32000), the
 same depth, and run the same forced-token workload through the serving engine
 (``lumen.serve.trace.TraceReplay``: the engine's input builder, block manager, state slots,
@@ -93,6 +95,40 @@ def fanopel_config(width: int, depth: int = 4):
                        rms_norm_eps=1e-6, residual_mult=0.5, intermediate_size=0,
                        num_attention_heads=0, num_key_value_heads=0, max_position_embeddings=4096,
                        eos_token_id=-1, name=f"fanopel-w{W}", layer_specs=[layer] * depth)
+
+
+def foderax_config(width: int, depth_groups: int = 1):
+    """One of each layer kind per group of four: a parallel layer (sigmoid-weight attention with
+    heads of 128 beside a minGRU of the model's width), latent attention at Dalavik's shapes
+    (latent 512, query latent 3/4 of the width), differential attention (two maps of 128 per head
+    over values of 256) and a second one that borrows the first one's caches; 16 experts of FFN
+    width 2.75 / 4 x model width in 4 groups of which 2 are kept, top 4 (Fanopel's shapes)."""
+    from ..models.config import ModelConfig
+
+    W = width
+    H = W // 128
+    mlp = {"kind": "moe", "expert": {"ff": int(2.75 * W) // 4},
+           "router": {"experts": 16, "top": 4, "groups": {"count": 4, "keep": 2}}}
+    layers = []
+    for g in range(depth_groups):
+        dif = {"heads": H // 2, "kv_heads": max(1, H // 8), "dim": 128, "vdim": 256,
+               "scale": 128 ** -0.5, "diff": 0.25, "rot": {"base": 500000.0, "dims": 128}}
+        layers += [
+            {"type": "parallel", "mlp": mlp, "mixer": {
+                "left": {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128,
+                         "scale": 128 ** -0.5, "rot": {"base": 20000.0, "dims": 64}},
+                "right": {"width": W}, "left_scale": 0.7, "right_scale": 0.4}},
+            {"type": "latent_attention", "mlp": mlp,
+             "mixer": {"heads": H, "dim": 128, "vdim": 128, "kv_rank": 512, "q_rank": 3 * W // 4,
+                       "scale": 128 ** -0.5}},
+            {"type": "attention", "mlp": mlp, "mixer": dict(dif)},
+            {"type": "attention", "mlp": mlp, "mixer": dict(dif, kv_from=4 * g + 2)}]
+    return ModelConfig(arch="foderax", vocab_size=32000, hidden_size=W,
+                       num_hidden_layers=len(layers), rms_norm_eps=1e-6,
+                       embedding_scale=float(W) ** 0.5, logit_softcap=30.0, intermediate_size=0,
+                       num_attention_heads=0, num_key_value_heads=0,
+                       max_position_embeddings=1 << 20, eos_token_id=-1, tie_word_embeddings=True,
+                       name=f"foderax-w{W}", layer_specs=layers)
 
 
 def gedatar_attention_moe_config(width: int, depth: int = 4):
@@ -187,12 +223,15 @@ def run_hybrid_bench(args) -> list:
     assert native() is not None, native_error()
     rows = []
     family = getattr(args, "hybrid_family", "gedatar")
-    make = {"gedatar": gedatar_config, "dalavik": dalavik_config, "fanopel": fanopel_config}[family]
+    make = {"gedatar": gedatar_config, "dalavik": dalavik_config, "fanopel": fanopel_config,
+            "foderax": foderax_config}[family]
     for width in [int(w) for w in str(args.hybrid_widths).split(",")]:
         gcfg = make(width)
         beside = [llama_config(width, gcfg.num_hidden_layers)]
         if family == "fanopel":
             beside.insert(0, gedatar_attention_moe_config(width, gcfg.num_hidden_layers))
+        if family == "foderax":
+            beside = [dalavik_config(width), fanopel_config(width, gcfg.num_hidden_layers)] + beside
         for cfg in [gcfg] + beside:
             for batch in [int(b) for b in str(args.hybrid_batch).split(",")]:
                 r = run_one(cfg, batch, args.hybrid_prompt, args.hybrid_decode_steps, 3, dev)
@@ -212,6 +251,11 @@ def run_hybrid_bench(args) -> list:
             gd = by[(w, b, "gedatar")]
             row["prefill_vs_gedatar"] = round(r["prefill_tok_s"] / gd["prefill_tok_s"], 3)
             row["decode_vs_gedatar"] = round(r["decode_tok_s"] / gd["decode_tok_s"], 3)
+        if family == "foderax":
+            for other in ("dalavik", "fanopel"):
+                o = by[(w, b, other)]
+                row[f"prefill_vs_{other}"] = round(r["prefill_tok_s"] / o["prefill_tok_s"], 3)
+                row[f"decode_vs_{other}"] = round(r["decode_tok_s"] / o["decode_tok_s"], 3)
         summ.append(row)
     metric = "hybrid" if family == "gedatar" else family
     print(json.dumps({"metric": f"{metric}_vs_llama_tokens_per_s", "dtype": "bf16",
