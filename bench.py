@@ -496,6 +496,9 @@ def main():
                          "one GPU (lumen/bench/hybrid_bench.py)")
     ap.add_argument("--hybrid_family", default="gedatar",
                     choices=["gedatar", "dalavik", "fanopel", "foderax"])
+    ap.add_argument("--hybrid_only", action="store_true",
+                    help="with --hybrid: run the family alone, without the models beside it "
+                         "(a kernel trace of one design)")
     ap.add_argument("--hybrid_widths", default="2048,4096")
     ap.add_argument("--hybrid_batch", default="8,64", help="sequences per step (comma list)")
     ap.add_argument("--hybrid_prompt", type=int, default=512)

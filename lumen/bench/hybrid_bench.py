@@ -232,6 +232,8 @@ def run_hybrid_bench(args) -> list:
             beside.insert(0, gedatar_attention_moe_config(width, gcfg.num_hidden_layers))
         if family == "foderax":
             beside = [dalavik_config(width), fanopel_config(width, gcfg.num_hidden_layers)] + beside
+        if getattr(args, "hybrid_only", False):
+            beside = []
         for cfg in [gcfg] + beside:
             for batch in [int(b) for b in str(args.hybrid_batch).split(",")]:
                 r = run_one(cfg, batch, args.hybrid_prompt, args.hybrid_decode_steps, 3, dev)
@@ -240,6 +242,8 @@ def run_hybrid_bench(args) -> list:
                 print(json.dumps(r), flush=True)
     by = {(r["width"], r["batch"], r["model"].split("-")[0]): r for r in rows}
     summ = []
+    if getattr(args, "hybrid_only", False):
+        return rows
     for (w, b, kind), r in list(by.items()):
         if kind != family:
             continue
