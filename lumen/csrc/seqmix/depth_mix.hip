@@ -14,7 +14,7 @@
 //   sm_min_gru        S_t = (1 - z_t) S_(t-1) + z_t c_t per channel over the rows of a segment,
 //                     z = sigmoid(zl + b_z), c = u + shift (u >= 0) | sigmoid(u), u = xl + b_x,
 //                     out = S_t * silu(gl); the fp32 state lives in [slots][width] across steps.
-//                     Long segments are cut into chunks: pass 1 reduces every chunk to its affine
+//                     Prompt portions are cut into chunks: pass 1 reduces every chunk to its affine
 //                     map S -> A S + B, pass 2 walks the chunks' maps (few) and replays each chunk
 //                     from its true start state -- a row's result is the same fp32 recurrence
 //                     whichever way the step was cut, up to the rounding of A S + B.
@@ -193,61 +193,105 @@ min_gru_seq_kernel(const GruArgs<T> a) {
   *sp = S;
 }
 
-// chunked form, pass 1: chunk -> (A, B) with S_end = A S_begin + B
+// chunked form: a tile of `chunk` rows is cut into kSub sub-chunks (grid z), each a short serial
+// walk, so that a step's prompt rows keep thousands of waves busy.
+constexpr int kSub = 4;
+constexpr int kGruUnroll = 8;
+
+template <typename T>
+struct GruSpan {
+  int seg, ra, rb, s0, s1, q, q_first;       // rows [ra, rb) of segment rows [s0, s1); map index
+  __device__ __forceinline__ GruSpan(const GruArgs<T>& a) {
+    const int ch = blockIdx.y, z = blockIdx.z, sub = (a.chunk + kSub - 1) / kSub;
+    seg = a.tiles[2 * ch];
+    const int r0 = a.tiles[2 * ch + 1];
+    s0 = a.cu[seg];
+    s1 = a.cu[seg + 1];
+    const int r1 = min(r0 + a.chunk, s1);
+    ra = min(r0 + z * sub, r1);
+    rb = min(ra + sub, r1);
+    q = ch * kSub + z;
+    q_first = (ch - (r0 - s0) / a.chunk) * kSub;
+  }
+};
+
+// pass 1: sub-chunk -> (A, B) with S_end = A S_begin + B; rows are loaded kGruUnroll at a time
+// before the serial updates, so the walk is not one memory round trip per row
 template <typename T>
 __global__ void __launch_bounds__(64)
 min_gru_reduce_kernel(const GruArgs<T> a) {
-  const int ch = blockIdx.y, c = blockIdx.x * 64 + threadIdx.x;
+  const int c = blockIdx.x * 64 + threadIdx.x;
   if (c >= a.width) return;
-  const int seg = a.tiles[2 * ch], r0 = a.tiles[2 * ch + 1];
-  const int r1 = min(r0 + a.chunk, a.cu[seg + 1]);
+  const GruSpan<T> sp(a);
+  if (sp.rb <= sp.ra) return;
   const float bz = a.bz[c], bx = a.bx[c];
   float A = 1.f, B = 0.f;
-  for (int r = r0; r < r1; ++r) {
-    float z, cand;
-    gru_gates(a, r, c, bz, bx, z, cand);
-    A *= 1.f - z;
-    B = (1.f - z) * B + z * cand;
+  for (int r = sp.ra; r < sp.rb; r += kGruUnroll) {
+    float zl[kGruUnroll], xl[kGruUnroll];
+#pragma unroll
+    for (int u = 0; u < kGruUnroll; ++u) {
+      const T* p = a.zxg + (long long)min(r + u, sp.rb - 1) * a.ld;
+      zl[u] = to_f32(p[c]);
+      xl[u] = to_f32(p[a.width + c]);
+    }
+#pragma unroll
+    for (int u = 0; u < kGruUnroll; ++u) {
+      if (r + u < sp.rb) {
+        const float z = sigmoid_f(zl[u] + bz), uu = xl[u] + bx;
+        const float cand = uu >= 0.f ? uu + a.shift : sigmoid_f(uu);
+        A *= 1.f - z;
+        B = (1.f - z) * B + z * cand;
+      }
+    }
   }
-  a.ab[((long long)ch * 2) * a.width + c] = A;
-  a.ab[((long long)ch * 2 + 1) * a.width + c] = B;
+  a.ab[((long long)sp.q * 2) * a.width + c] = A;
+  a.ab[((long long)sp.q * 2 + 1) * a.width + c] = B;
 }
 
-// pass 2: a chunk's start state from the maps of the chunks before it in its segment, then the
-// chunk replayed; the segment's last chunk stores the state
+// pass 2: a sub-chunk's start state from the maps of those before it in its segment, then the
+// sub-chunk replayed; the segment's last one parks the end state in its own map's place
 template <typename T>
 __global__ void __launch_bounds__(64)
 min_gru_replay_kernel(const GruArgs<T> a) {
-  const int ch = blockIdx.y, c = blockIdx.x * 64 + threadIdx.x;
+  const int c = blockIdx.x * 64 + threadIdx.x;
   if (c >= a.width) return;
-  const int seg = a.tiles[2 * ch], r0 = a.tiles[2 * ch + 1];
-  const int s0 = a.cu[seg], s1 = a.cu[seg + 1];
-  const int r1 = min(r0 + a.chunk, s1);
-  float* sp = a.state + (long long)a.slot[seg] * a.width + c;
-  float S = a.start[seg] > 0 ? *sp : 0.f;
-  const int before = (r0 - s0) / a.chunk;           // chunks of this segment ahead of this one
-  for (int k = ch - before; k < ch; ++k)
+  const GruSpan<T> sp(a);
+  if (sp.rb <= sp.ra) return;
+  float S = a.start[sp.seg] > 0 ? a.state[(long long)a.slot[sp.seg] * a.width + c] : 0.f;
+  for (int k = sp.q_first; k < sp.q; ++k)
     S = a.ab[((long long)k * 2) * a.width + c] * S + a.ab[((long long)k * 2 + 1) * a.width + c];
   const float bz = a.bz[c], bx = a.bx[c];
-  for (int r = r0; r < r1; ++r) {
-    float z, cand;
-    gru_gates(a, r, c, bz, bx, z, cand);
-    S = (1.f - z) * S + z * cand;
-    const float g = to_f32(a.zxg[(long long)r * a.ld + 2 * a.width + c]);
-    a.out[(long long)r * a.width + c] = from_f32<T>(S * silu_f(g));
+  for (int r = sp.ra; r < sp.rb; r += kGruUnroll) {
+    float zl[kGruUnroll], xl[kGruUnroll], gl[kGruUnroll];
+#pragma unroll
+    for (int u = 0; u < kGruUnroll; ++u) {
+      const T* p = a.zxg + (long long)min(r + u, sp.rb - 1) * a.ld;
+      zl[u] = to_f32(p[c]);
+      xl[u] = to_f32(p[a.width + c]);
+      gl[u] = to_f32(p[2 * a.width + c]);
+    }
+#pragma unroll
+    for (int u = 0; u < kGruUnroll; ++u) {
+      if (r + u < sp.rb) {
+        const float z = sigmoid_f(zl[u] + bz), uu = xl[u] + bx;
+        const float cand = uu >= 0.f ? uu + a.shift : sigmoid_f(uu);
+        S = (1.f - z) * S + z * cand;
+        a.out[(long long)(r + u) * a.width + c] = from_f32<T>(S * silu_f(gl[u]));
+      }
+    }
   }
-  if (r1 == s1) a.ab[((long long)ch * 2) * a.width + c] = S;   // parked: stored once all have read
+  if (sp.rb == sp.s1) a.ab[((long long)sp.q * 2) * a.width + c] = S;   // stored once all have read
 }
 
-// pass 3: the parked end states into the slots (after every chunk has read its start state)
+// pass 3: the parked end states into the slots (after every sub-chunk has read its start state)
 template <typename T>
 __global__ void __launch_bounds__(64)
-min_gru_store_kernel(const GruArgs<T> a, int n_chunks) {
-  const int ch = blockIdx.y, c = blockIdx.x * 64 + threadIdx.x;
-  if (c >= a.width || ch >= n_chunks) return;
-  const int seg = a.tiles[2 * ch], r0 = a.tiles[2 * ch + 1];
-  if (r0 + a.chunk < a.cu[seg + 1]) return;         // not the segment's last chunk
-  a.state[(long long)a.slot[seg] * a.width + c] = a.ab[((long long)ch * 2) * a.width + c];
+min_gru_store_kernel(const GruArgs<T> a) {
+  const int c = blockIdx.x * 64 + threadIdx.x;
+  if (c >= a.width) return;
+  const GruSpan<T> sp(a);
+  if (sp.rb <= sp.ra || sp.rb != sp.s1) return;
+  a.state[(long long)a.slot[sp.seg] * a.width + c] = a.ab[((long long)sp.q * 2) * a.width + c];
 }
 
 // one wave per (row, head)
@@ -362,7 +406,10 @@ hipError_t sm_rotary_write(int dt, void* z, long long ld, const int* positions,
 // tiles == nullptr: one thread per channel walks a whole segment (segments 0 .. n_seg - 1 of
 // cu / slot / start; rows are absolute).  Else the chunked form over the n_chunks chunks listed
 // in `tiles` ([n_chunks][2] = segment, first row; a segment's chunks consecutive, `chunk` rows
-// each from the segment's first row on), with `ab` a scratch of n_chunks * 2 * width floats.
+// each from the segment's first row on), with `ab` a scratch of n_chunks * sm_min_gru_sub() * 2 *
+// width floats.
+int sm_min_gru_sub() { return kSub; }
+
 hipError_t sm_min_gru(int dt, const void* zxg, long long ld, const float* bz, const float* bx,
                       float* state, void* out, const int* cu, const int* slot, const int* start,
                       int n_seg, int width, float shift, float* ab, const int* tiles,
@@ -378,9 +425,9 @@ hipError_t sm_min_gru(int dt, const void* zxg, long long ld, const float* bz, co
       min_gru_seq_kernel<TT><<<dim3(gx, n_seg), 64, 0, st>>>(a);                                \
     } else {                                                                                    \
       if (ab == nullptr || chunk < 1) return hipErrorInvalidValue;                              \
-      min_gru_reduce_kernel<TT><<<dim3(gx, n_chunks), 64, 0, st>>>(a);                          \
-      min_gru_replay_kernel<TT><<<dim3(gx, n_chunks), 64, 0, st>>>(a);                          \
-      min_gru_store_kernel<TT><<<dim3(gx, n_chunks), 64, 0, st>>>(a, n_chunks);                 \
+      min_gru_reduce_kernel<TT><<<dim3(gx, n_chunks, kSub), 64, 0, st>>>(a);                    \
+      min_gru_replay_kernel<TT><<<dim3(gx, n_chunks, kSub), 64, 0, st>>>(a);                    \
+      min_gru_store_kernel<TT><<<dim3(gx, n_chunks, kSub), 64, 0, st>>>(a);                     \
     }                                                                                           \
   }
   SM_DISPATCH(dt, CALL)

@@ -79,6 +79,8 @@ def _load():
         lib.sm_row_attn_lds.restype = ctypes.c_int
         lib.sm_latent_attn_ok.argtypes = [ctypes.c_int] * 5
         lib.sm_latent_attn_ok.restype = ctypes.c_int
+        lib.sm_min_gru_sub.argtypes = []
+        lib.sm_min_gru_sub.restype = ctypes.c_int
         _lib = lib
     except Exception as e:  # pragma: no cover - depends on build state
         _err = e
@@ -122,6 +124,11 @@ def row_attn_lds(HB: int, Dk: int) -> int:
 def latent_attn_ok(dt: int, Dv: int, Dk: int, D1: int, bs: int) -> bool:
     """Does the matrix-core latent attention have a kernel for these sizes?"""
     return bool(_load().sm_latent_attn_ok(dt, Dv, Dk, D1, bs))
+
+
+def min_gru_sub() -> int:
+    """Sub-chunks the minGRU scan cuts a tile of prompt rows into (sizes its scratch)."""
+    return int(_load().sm_min_gru_sub())
 
 
 def _arg(kind, v):

@@ -180,7 +180,7 @@ def min_gru_scan(zxg: torch.Tensor, b_z: torch.Tensor, b_x: torch.Tensor, state:
     fused projection's rows, unit column stride), biases [width] fp32 -> [T, width] in zxg's dtype,
     ready for the output projection; ``state`` [slots, width] fp32 moves on by the step's rows (a
     segment that starts at position 0 begins from zero whatever its slot holds)."""
-    from ._seqmix import DT, call, use_seqmix
+    from ._seqmix import DT, call, min_gru_sub, use_seqmix
 
     if zxg.shape[1] < 3 * width:
         raise ValueError(f"zxg has {zxg.shape[1]} columns, expected at least {3 * width}")
@@ -196,7 +196,7 @@ def min_gru_scan(zxg: torch.Tensor, b_z: torch.Tensor, b_x: torch.Tensor, state:
     Tp = seg.tile_rows if seg.q_tiles is not None else 0
     if Tp:
         n = seg.q_tiles.shape[0]
-        ab = torch.empty(n * 2 * width, dtype=torch.float32, device=zxg.device)
+        ab = torch.empty(n * min_gru_sub() * 2 * width, dtype=torch.float32, device=zxg.device)
         call("sm_min_gru", DT[zxg.dtype], zxg, zxg.stride(0), b_z, b_x, state, out, seg.cu,
              seg.slot, seg.start, 0, width, float(shift), ab, seg.q_tiles, n, seg.tile_size)
     if T > Tp:

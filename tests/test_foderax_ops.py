@@ -182,7 +182,7 @@ def test_min_gru_candidate_is_continuous_at_zero(device, dtype):
     out = min_gru_scan(zxg, zero, zero, state, seg, width, 0.5)
     uu = zxg[0, width:2 * width].cpu().to(F64)
     want = torch.where(uu >= 0, uu + 0.5, torch.sigmoid(uu)) * 40.0    # silu(40) = 40
-    close(out[0], want, dtype, scale=40.0)
+    close(out[0], want, dtype, scale=float(want.abs().max()))
 
 
 # ---- attention whose weights are sigmoids --------------------------------------------------------------
