@@ -29,7 +29,7 @@ namespace {
 
 constexpr int kThreads = 256;
 
-template <typename T>
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(kThreads)
 embed_scaled_kernel(const T* __restrict__ table, const long long* __restrict__ tokens,
                     float* __restrict__ out, int W, int V, float scale) {
@@ -37,7 +37,17 @@ embed_scaled_kernel(const T* __restrict__ table, const long long* __restrict__ t
   tok = tok < 0 ? 0 : (tok >= V ? V - 1 : tok);
   const T* src = table + tok * W;
   float* dst = out + (long long)blockIdx.x * W;
-  for (int c = threadIdx.x; c < W; c += kThreads) dst[c] = to_f32(src[c]) * scale;
+  if constexpr (VEC) {
+    for (int c = threadIdx.x * 4; c < W; c += kThreads * 4) {
+      float v[4];
+      load4<T>(src + c, v);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] *= scale;
+      store4<float>(dst + c, v);
+    }
+  } else {
+    for (int c = threadIdx.x; c < W; c += kThreads) dst[c] = to_f32(src[c]) * scale;
+  }
 }
 
 template <typename TY>
@@ -294,8 +304,8 @@ min_gru_store_kernel(const GruArgs<T> a) {
   a.state[(long long)a.slot[sp.seg] * a.width + c] = a.ab[((long long)sp.q * 2) * a.width + c];
 }
 
-// one wave per (row, head)
-template <typename T>
+// one wave per (row, head); VEC: a lane owns 4 consecutive channels of every 256
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(256)
 diff_combine_kernel(const T* __restrict__ av, const T* __restrict__ gate, long long gater,
                     T* __restrict__ out, int Tn, int G, int rep, int Dv, float lam,
@@ -309,19 +319,48 @@ diff_combine_kernel(const T* __restrict__ av, const T* __restrict__ gate, long l
   const T* a1 = av + ((t * G + g) * 2 * rep + r) * Dv;
   const T* a2 = a1 + (long long)rep * Dv;
   float o[8], sq = 0.f;                               // Dv <= 512
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const int d = lane + 64 * e;
-    o[e] = d < Dv ? to_f32(a1[d]) - lam * to_f32(a2[d]) : 0.f;
-    sq += o[e] * o[e];
-  }
-  const float inv = out_scale / sqrtf(wave_sum(sq) / (float)Dv + eps);
   T* op = out + (t * H + h) * Dv;
   const T* gp = gate ? gate + t * gater + (long long)h * Dv : nullptr;
+  if constexpr (VEC) {
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const int d = lane + 64 * e;
-    if (d < Dv) op[d] = from_f32<T>(o[e] * inv * (gp ? sigmoid_f(to_f32(gp[d])) : 1.f));
+    for (int b = 0; b < 2; ++b) {
+      const int d = 4 * lane + 256 * b;
+      float x1[4] = {0.f, 0.f, 0.f, 0.f}, x2[4] = {0.f, 0.f, 0.f, 0.f};
+      if (d < Dv) {
+        load4<T>(a1 + d, x1);
+        load4<T>(a2 + d, x2);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        o[4 * b + e] = x1[e] - lam * x2[e];
+        sq += o[4 * b + e] * o[4 * b + e];
+      }
+    }
+    const float inv = out_scale / sqrtf(wave_sum(sq) / (float)Dv + eps);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int d = 4 * lane + 256 * b;
+      if (d < Dv) {
+        float gv[4] = {0.f, 0.f, 0.f, 0.f}, r[4];
+        if (gp) load4<T>(gp + d, gv);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = o[4 * b + e] * inv * (gp ? sigmoid_f(gv[e]) : 1.f);
+        store4<T>(op + d, r);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int d = lane + 64 * e;
+      o[e] = d < Dv ? to_f32(a1[d]) - lam * to_f32(a2[d]) : 0.f;
+      sq += o[e] * o[e];
+    }
+    const float inv = out_scale / sqrtf(wave_sum(sq) / (float)Dv + eps);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int d = lane + 64 * e;
+      if (d < Dv) op[d] = from_f32<T>(o[e] * inv * (gp ? sigmoid_f(to_f32(gp[d])) : 1.f));
+    }
   }
 }
 
@@ -346,7 +385,12 @@ extern "C" {
 hipError_t sm_embed_scaled(int dt, const void* table, const long long* tokens, float* out, int T,
                            int W, int V, float scale, hipStream_t st) {
   if (T == 0) return hipSuccess;
-#define CALL(TT) embed_scaled_kernel<TT><<<T, kThreads, 0, st>>>((const TT*)table, tokens, out, W, V, scale)
+  const bool vec = W % 4 == 0 && (uintptr_t)table % 16 == 0 && (uintptr_t)out % 16 == 0;
+#define CALL(TT)                                                                                \
+  if (vec) embed_scaled_kernel<TT, true><<<T, kThreads, 0, st>>>((const TT*)table, tokens, out, \
+                                                                 W, V, scale);                  \
+  else embed_scaled_kernel<TT, false><<<T, kThreads, 0, st>>>((const TT*)table, tokens, out, W, \
+                                                              V, scale)
   SM_DISPATCH(dt, CALL)
 #undef CALL
   return hipGetLastError();
@@ -441,7 +485,13 @@ hipError_t sm_diff_combine(int dt, const void* av, const void* gate, long long g
   if (T == 0) return hipSuccess;
   if (Dv < 1 || Dv > 512 || G < 1 || rep < 1) return hipErrorInvalidValue;
   const long long waves = (long long)T * G * rep;
-#define CALL(TT) diff_combine_kernel<TT><<<(unsigned)((waves + 3) / 4), 256, 0, st>>>((const TT*)av, (const TT*)gate, gater, (TT*)out, T, G, rep, Dv, lam, out_scale, eps)
+  const bool vec = Dv % 4 == 0 && (uintptr_t)av % 16 == 0 && (uintptr_t)out % 16 == 0 &&
+                   (gate == nullptr || ((uintptr_t)gate % 16 == 0 && gater % 4 == 0));
+#define CALL(TT)                                                                                \
+  if (vec) diff_combine_kernel<TT, true><<<(unsigned)((waves + 3) / 4), 256, 0, st>>>(          \
+      (const TT*)av, (const TT*)gate, gater, (TT*)out, T, G, rep, Dv, lam, out_scale, eps);     \
+  else diff_combine_kernel<TT, false><<<(unsigned)((waves + 3) / 4), 256, 0, st>>>(             \
+      (const TT*)av, (const TT*)gate, gater, (TT*)out, T, G, rep, Dv, lam, out_scale, eps)
   SM_DISPATCH(dt, CALL)
 #undef CALL
   return hipGetLastError();

@@ -4,8 +4,12 @@
 //   s(i, j) = cap * tanh(q_i . k_j * scale / cap) - slope_h * (i - j)
 //   row i sees key j when j <= i and (window == 0 or i - j < window or j < keep)
 //   o_i = sigmoid(gate[i, h]) * sum_j softmax_j(s(i, j)) v_j
+// or, with a per-head bias `sigb`, weights that are sigmoids and are not normalised:
+//   o_i = sum_j sigmoid(s(i, j) + sigb_h) v_j
 // q arrives as the projection left it (already normed where the design norms it), the key cache
-// holds what the scores read and the value cache what is summed; both are [blocks][bs][G][D].
+// [blocks][bs][G][D] holds what the scores read and the value cache [blocks][bs][G / vdiv][DV]
+// what is summed: the value size may differ from the key size, and `vdiv` consecutive key heads
+// may share one value head (several score maps over the same values).
 //
 // A workgroup of NW waves takes 32 * NW consecutive rows of ONE segment and one query head.  The
 // keys the tile can see are visited 32 at a time: first the tiles of the kept keys that lie below
@@ -67,8 +71,8 @@ __device__ __forceinline__ float tanh_exp(float x) { return 1.f - 2.f / (1.f + _
 template <typename T>
 struct WinTileArgs {
   const T* q; long long ldq;                 // rows [T][>= H * D]
-  const T* kc; const T* vc;                  // [blocks][bs][G][D] each
-  T* out;                                    // [T][H][D]
+  const T* kc; const T* vc;                  // [blocks][bs][G][D], [blocks][bs][G / vdiv][DV]
+  T* out;                                    // [T][H][DV]
   const T* gate; long long gater;            // gate logits [T][H], row stride (nullable)
   const int* tables; int maxb;
   const int* tiles; const int* cu; const int* start;
@@ -76,18 +80,22 @@ struct WinTileArgs {
   float scale, softcap;
   const float* slopes;                       // [H] (nullable)
   int window, keep;
+  const float* sigb; int vdiv;               // sigmoid weights' bias [H] (nullable); key heads per value head
 };
 
-template <typename T, int D, int NW>
-__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(D <= 128 ? 2 : 1)))
+template <typename T, int D, int DV, int NW>
+__global__ void __launch_bounds__(64 * NW)
+    __attribute__((amdgpu_waves_per_eu((D <= 128 && DV <= 128) ? 2 : 1)))
 win_tile_attn_kernel(const WinTileArgs<T> a) {
-  constexpr int QT = 32 * NW, LK = D + 8, LT = 40, NV = D / 8;
+  constexpr int QT = 32 * NW, LK = D + 8, LT = 40, NV = D / 8, NVV = DV / 8;
   __shared__ __align__(16) T s_k[32 * LK];    // key tile, row-major
-  __shared__ __align__(16) T s_t[D * LT];     // value tile, transposed [d][key]
+  __shared__ __align__(16) T s_t[DV * LT];    // value tile, transposed [d][key]
   constexpr int kTbl = 512;                   // block-table entries of the window's keys, in LDS
   __shared__ int s_tbl[kTbl];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c = lane & 31, hi = lane >> 5;
   const int hd = blockIdx.y, g = hd / (a.H / a.G);
+  const int Gv = a.G / a.vdiv, gv = g / a.vdiv;
+  const float sbias = a.sigb != nullptr ? a.sigb[hd] : 0.f;
   // tiles are listed in row order, so later tiles see more keys: issue them first
   const int tix = gridDim.x - 1 - blockIdx.x;
   const int sg = a.tiles[2 * tix], row0 = a.tiles[2 * tix + 1];
@@ -128,17 +136,23 @@ win_tile_attn_kernel(const WinTileArgs<T> a) {
   __syncthreads();
 
   float m = -INFINITY, l = 0.f;
-  f32x16 O[D / 32];
+  f32x16 O[DV / 32];
 #pragma unroll
-  for (int db = 0; db < D / 32; ++db)
+  for (int db = 0; db < DV / 32; ++db)
 #pragma unroll
     for (int r = 0; r < 16; ++r) O[db][r] = 0.f;
 
   // staging: one item = 4 consecutive keys x 8 channels of the key cache AND of the value cache
   // (four 16-byte loads each); the row-major image takes the keys as they are, the transposed
   // image takes eight 8-byte stores of 4 values each (transposed in registers)
-  constexpr int NT = 64 * NW, ITEMS = (D + NT - 1) / NT;
-  uint4 pk[ITEMS][4], pv[ITEMS][4];
+  constexpr int NT = 64 * NW, ITEMS = (D + NT - 1) / NT, ITEMS_V = (DV + NT - 1) / NT;
+  uint4 pk[ITEMS][4], pv[ITEMS_V][4];
+  auto cache_row = [&](int j) -> long long {
+    const int jb = bshift >= 0 ? j >> bshift : j / bs, jo = j - jb * bs;
+    const int bi = jb - b_first;
+    const int blk = (bi >= 0 && bi < kTbl) ? s_tbl[bi] : tbl[jb];
+    return (long long)blk * bs + jo;
+  };
   auto prefetch = [&](int k0) {
 #pragma unroll
     for (int it = 0; it < ITEMS; ++it) {
@@ -149,15 +163,22 @@ win_tile_attn_kernel(const WinTileArgs<T> a) {
         for (int x = 0; x < 4; ++x) {
           const int j = k0 + 4 * kq + x;
           pk[it][x] = make_uint4(0, 0, 0, 0);
+          if (j <= kend)
+            pk[it][x] = *reinterpret_cast<const uint4*>(a.kc + (cache_row(j) * a.G + g) * D + 8 * part);
+        }
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < ITEMS_V; ++it) {
+      const int item = tid + it * NT;
+      if (item < DV) {
+        const int kq = item / NVV, part = item % NVV;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          const int j = k0 + 4 * kq + x;
           pv[it][x] = make_uint4(0, 0, 0, 0);
-          if (j <= kend) {
-            const int jb = bshift >= 0 ? j >> bshift : j / bs, jo = j - jb * bs;
-            const int bi = jb - b_first;
-            const int blk = (bi >= 0 && bi < kTbl) ? s_tbl[bi] : tbl[jb];
-            const long long off = (((long long)blk * bs + jo) * a.G + g) * D + 8 * part;
-            pk[it][x] = *reinterpret_cast<const uint4*>(a.kc + off);
-            pv[it][x] = *reinterpret_cast<const uint4*>(a.vc + off);
-          }
+          if (j <= kend)
+            pv[it][x] = *reinterpret_cast<const uint4*>(a.vc + (cache_row(j) * Gv + gv) * DV + 8 * part);
         }
       }
     }
@@ -171,6 +192,13 @@ win_tile_attn_kernel(const WinTileArgs<T> a) {
 #pragma unroll
         for (int x = 0; x < 4; ++x)
           *reinterpret_cast<uint4*>(&s_k[(4 * kq + x) * LK + 8 * part]) = pk[it][x];
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < ITEMS_V; ++it) {
+      const int item = tid + it * NT;
+      if (item < DV) {
+        const int kq = item / NVV, part = item % NVV;
         const unsigned w0[4] = {pv[it][0].x, pv[it][0].y, pv[it][0].z, pv[it][0].w};
         const unsigned w1[4] = {pv[it][1].x, pv[it][1].y, pv[it][1].z, pv[it][1].w};
         const unsigned w2[4] = {pv[it][2].x, pv[it][2].y, pv[it][2].z, pv[it][2].w};
@@ -228,24 +256,30 @@ win_tile_attn_kernel(const WinTileArgs<T> a) {
         sc[r] = seen ? sc[r] : -INFINITY;
       }
     }
+    if (a.sigb != nullptr) {
+      // weights as they are: a hidden key's -inf gives 1 / (1 + e^inf) = 0
 #pragma unroll
-    for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, sc[r]);
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-    const float mn = fmaxf(m, mloc);
-    const float ms = mn == -INFINITY ? 0.f : mn;
-    // (v_exp_f32: this kernel serves 16-bit dtypes only, the weights are rounded to ~16 bits)
-    const float corr = __expf(m - ms);
-    float psum = 0.f;
+      for (int r = 0; r < 16; ++r) sc[r] = 1.f / (1.f + __expf(-(sc[r] + sbias)));
+    } else {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { sc[r] = __expf(sc[r] - ms); psum += sc[r]; }
-    psum += __shfl_xor(psum, 32, 64);
-    l = l * corr + psum;
-    m = mn;
-    if (__any(corr != 1.f)) {              // the running max moved for some query of the wave
+      for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, sc[r]);
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+      const float mn = fmaxf(m, mloc);
+      const float ms = mn == -INFINITY ? 0.f : mn;
+      // (v_exp_f32: this kernel serves 16-bit dtypes only, the weights are rounded to ~16 bits)
+      const float corr = __expf(m - ms);
+      float psum = 0.f;
 #pragma unroll
-      for (int db = 0; db < D / 32; ++db)
+      for (int r = 0; r < 16; ++r) { sc[r] = __expf(sc[r] - ms); psum += sc[r]; }
+      psum += __shfl_xor(psum, 32, 64);
+      l = l * corr + psum;
+      m = mn;
+      if (__any(corr != 1.f)) {            // the running max moved for some query of the wave
 #pragma unroll
-        for (int r = 0; r < 16; ++r) O[db][r] *= corr;
+        for (int db = 0; db < DV / 32; ++db)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) O[db][r] *= corr;
+      }
     }
 #pragma unroll
     for (int s2 = 0; s2 < 2; ++s2) {
@@ -261,7 +295,7 @@ win_tile_attn_kernel(const WinTileArgs<T> a) {
       const uint4 bh = make_uint4(ph[0], ph[1], ph[2], ph[3]);
       const uint4 bl = make_uint4(pl[0], pl[1], pl[2], pl[3]);
 #pragma unroll
-      for (int db = 0; db < D / 32; ++db) {
+      for (int db = 0; db < DV / 32; ++db) {
         const int row = 32 * db + c, sw = (row >> 3) & 7;     // undo the store's permutation
         const T* tp = &s_t[row * LT];
         const uint2 a0 = *reinterpret_cast<const uint2*>(tp + 4 * ((4 * s2 + hi) ^ sw));
@@ -273,11 +307,11 @@ win_tile_attn_kernel(const WinTileArgs<T> a) {
     }
   }
   if (qv) {
-    float inv = 1.f / l;                   // l > 0: a row always sees its own key
+    float inv = a.sigb != nullptr ? 1.f : 1.f / l;   // l > 0: a row always sees its own key
     if (a.gate != nullptr) inv *= sigmoid_f(to_f32(a.gate[(long long)qrow * a.gater + hd]));
-    T* op = a.out + ((long long)qrow * a.H + hd) * D;
+    T* op = a.out + ((long long)qrow * a.H + hd) * DV;
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db)
+    for (int db = 0; db < DV / 32; ++db)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int d = 32 * db + 8 * j + 4 * hi;
@@ -289,19 +323,25 @@ win_tile_attn_kernel(const WinTileArgs<T> a) {
 }
 
 template <typename T>
-hipError_t launch_win_tiles(const WinTileArgs<T>& a, int ntiles, int D, int tile_rows,
+hipError_t launch_win_tiles(const WinTileArgs<T>& a, int ntiles, int D, int Dv, int tile_rows,
                             hipStream_t st) {
   const dim3 grid(ntiles, a.H);
-#define GO(DD)                                                        \
-  if (tile_rows == 128) win_tile_attn_kernel<T, DD, 4><<<grid, 256, 0, st>>>(a); \
-  else win_tile_attn_kernel<T, DD, 2><<<grid, 128, 0, st>>>(a)
-  switch (D) {
-    case 32: GO(32); break;
-    case 64: GO(64); break;
-    case 96: GO(96); break;
-    case 128: GO(128); break;
-    case 192: GO(192); break;
-    case 256: GO(256); break;
+#define GO(DD, DVV)                                                                          \
+  if (tile_rows == 128) win_tile_attn_kernel<T, DD, DVV, 4><<<grid, 256, 0, st>>>(a);        \
+  else win_tile_attn_kernel<T, DD, DVV, 2><<<grid, 128, 0, st>>>(a)
+  switch (D * 1024 + Dv) {
+    case 32 * 1024 + 32: GO(32, 32); break;
+    case 64 * 1024 + 64: GO(64, 64); break;
+    case 96 * 1024 + 96: GO(96, 96); break;
+    case 128 * 1024 + 128: GO(128, 128); break;
+    case 192 * 1024 + 192: GO(192, 192); break;
+    case 256 * 1024 + 256: GO(256, 256); break;
+    // values twice the key size (two score maps per head, or wide values)
+    case 32 * 1024 + 64: GO(32, 64); break;
+    case 48 * 1024 + 96: GO(48, 96); break;
+    case 64 * 1024 + 128: GO(64, 128); break;
+    case 96 * 1024 + 192: GO(96, 192); break;
+    case 128 * 1024 + 256: GO(128, 256); break;
     default: return hipErrorInvalidValue;
   }
 #undef GO
@@ -312,23 +352,26 @@ hipError_t launch_win_tiles(const WinTileArgs<T>& a, int ntiles, int D, int tile
 
 extern "C" {
 
-// 1 when sm_win_attn_tiles has a kernel for this dtype / head size
-int sm_win_attn_tiles_ok(int dt, int D) {
-  return (dt == kBF16 || dt == kF16) &&
-         (D == 32 || D == 64 || D == 96 || D == 128 || D == 192 || D == 256);
+// 1 when sm_win_attn_tiles has a kernel for this dtype / key size / value size
+int sm_win_attn_tiles_ok(int dt, int D, int Dv) {
+  if (dt != kBF16 && dt != kF16) return 0;
+  if (Dv == D) return D == 32 || D == 64 || D == 96 || D == 128 || D == 192 || D == 256;
+  return Dv == 2 * D && (D == 32 || D == 48 || D == 64 || D == 96 || D == 128);
 }
 
 // tiles: [ntiles, 2] int32 (segment, first row); every tile covers up to tile_rows (64 or 128)
 // rows of its segment.  q rows [T][>= H * D] with row stride ldq (a multiple of 8, 16-byte
-// aligned base); kc / vc [blocks][bs][G][D]; out [T][H][D] contiguous; gate (nullable) [T][H]
-// with row stride gater; slopes (nullable) fp32 [H]; window 0: plain causal attention.
+// aligned base); kc [blocks][bs][G][D], vc [blocks][bs][G / vdiv][Dv]; out [T][H][Dv] contiguous;
+// gate (nullable) [T][H] with row stride gater; slopes (nullable) fp32 [H]; window 0: plain causal
+// attention; sigb (nullable) fp32 [H]: sigmoid weights, not normalised.
 hipError_t sm_win_attn_tiles(int dt, const void* q, long long ldq, const void* kc, const void* vc,
                              void* out, const void* gate, long long gater, const int* tables,
                              int maxb, const int* tiles, int ntiles, const int* cu,
                              const int* start, int H, int G, int D, int bs, float scale,
                              float softcap, const float* slopes, int window, int keep,
-                             int tile_rows, hipStream_t st) {
+                             int tile_rows, int Dv, const float* sigb, int vdiv, hipStream_t st) {
   if (ntiles == 0) return hipSuccess;
+  if (vdiv < 1 || G % vdiv || !sm_win_attn_tiles_ok(dt, D, Dv)) return hipErrorInvalidValue;
   if (G < 1 || H % G || bs < 1 || window < 0 || keep < 0 || (ldq % 8) != 0 ||
       (uintptr_t)q % 16 || (uintptr_t)kc % 16 || (uintptr_t)vc % 16 || (uintptr_t)out % 8)
     return hipErrorInvalidValue;
@@ -337,8 +380,8 @@ hipError_t sm_win_attn_tiles(int dt, const void* q, long long ldq, const void* k
   {                                                                                            \
     WinTileArgs<TT> a{(const TT*)q, ldq, (const TT*)kc, (const TT*)vc, (TT*)out,               \
                       (const TT*)gate, gater, tables, maxb, tiles, cu, start, H, G, bs, scale, \
-                      softcap, slopes, window, keep};                                          \
-    return launch_win_tiles<TT>(a, ntiles, D, tile_rows, st);                                  \
+                      softcap, slopes, window, keep, sigb, vdiv};                              \
+    return launch_win_tiles<TT>(a, ntiles, D, Dv, tile_rows, st);                              \
   }
   if (dt == kBF16) CALL(bf16)
   if (dt == kF16) CALL(fp16)

@@ -41,7 +41,7 @@ SIGNATURES = {
     "sm_latent_attn": "i" "plli" "plli" "pl" "pi" "pll" "pi" "pp" "iii" "fffi" "ppp" "pl" "ipp",
     "sm_row_attn": "i" "plli" "plli" "pl" "pli" "pll" "pi" "pp" "iiiii" "fffi" "pppp" "piipl"
                    "pi" "ipp",
-    "sm_win_attn_tiles": "iplppppl" "pi" "pi" "pp" "iiii" "ff" "p" "iii",
+    "sm_win_attn_tiles": "iplppppl" "pi" "pi" "pp" "iiii" "ff" "p" "iii" "ipi",
     "sm_row_norm_write": "iplpppppiiif",
     "sm_layer_norm": "iippfppiif",
     "sm_embed_pos": "ipppppiiii",
@@ -73,7 +73,7 @@ def _load():
             fn.restype = ctypes.c_int
         lib.sm_chunk_attn_tiles_ok.argtypes = [ctypes.c_int, ctypes.c_int]
         lib.sm_chunk_attn_tiles_ok.restype = ctypes.c_int
-        lib.sm_win_attn_tiles_ok.argtypes = [ctypes.c_int, ctypes.c_int]
+        lib.sm_win_attn_tiles_ok.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int]
         lib.sm_win_attn_tiles_ok.restype = ctypes.c_int
         lib.sm_row_attn_lds.argtypes = [ctypes.c_int, ctypes.c_int]
         lib.sm_row_attn_lds.restype = ctypes.c_int
@@ -110,10 +110,10 @@ def tiles_ok(dt: int, D: int) -> bool:
     return bool(_load().sm_chunk_attn_tiles_ok(dt, D))
 
 
-def win_tiles_ok(dt: int, D: int) -> bool:
+def win_tiles_ok(dt: int, D: int, Dv: int = 0) -> bool:
     """Does the matrix-core prefill attention over paged key and value caches have a kernel for
-    this dtype code / head size?"""
-    return bool(_load().sm_win_attn_tiles_ok(dt, D))
+    this dtype code / key size / value size (0: the key size)?"""
+    return bool(_load().sm_win_attn_tiles_ok(dt, D, Dv or D))
 
 
 def row_attn_lds(HB: int, Dk: int) -> int:

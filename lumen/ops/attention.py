@@ -819,8 +819,8 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
 
     Three kernels serve it.  The prompt portions of a step (``seg.q_tiles``) go to the tiled
     matrix-core kernel of ``csrc/seqmix/window_attention.hip`` when the keys and values have caches
-    of their own, one query part, a head size it is built for, a 16-bit dtype and none of
-    temperature, logarithmic bias, head mixing or sink; the latent layout with ``vt`` goes to the
+    of their own, one query part, head sizes it is built for (values as wide as the keys or twice
+    as wide), a 16-bit dtype and none of temperature, logarithmic bias, head mixing or sink; the latent layout with ``vt`` goes to the
     latent kernel; every other row (decoded rows, fp32, other shapes) to the row kernel.  A row's
     result does not depend on which of them computed it beyond rounding."""
     from ._seqmix import DT, call, latent_attn_ok, use_seqmix, win_tiles_ok
@@ -881,15 +881,15 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
     Tp = 0
     if (seg.q_tiles is not None and seg.tile_rows > 0 and q2 is None and talk is None
             and sink is None and r1 is None and q_temp is None and vcache is not kcache
-            and sigmoid_bias is None and v_div == 1
-            and D1 == Dv and krow == G * D1 and vrow == G * Dv and win_tiles_ok(DT[q1.dtype], D1)
+            and krow == G * D1 and vrow == (G // v_div) * Dv and win_tiles_ok(DT[q1.dtype], D1, Dv)
             and q1.stride(1) == D1 and q1.stride(0) % 8 == 0 and q1.data_ptr() % 16 == 0
             and out.stride(1) == Dv and out.stride(0) == H * Dv and out.data_ptr() % 8 == 0):
         Tp = seg.tile_rows
         call("sm_win_attn_tiles", DT[q1.dtype], q1, q1.stride(0), kcache, vcache, out, gate,
              gate.stride(0) if gate is not None else 0, seg.tables, seg.tables.shape[1],
              seg.q_tiles, seg.q_tiles.shape[0], seg.cu, seg.start, H, G, D1, bs, scale,
-             float(softcap or 0.0), slopes, window, keep_first, seg.tile_size)
+             float(softcap or 0.0), slopes, window, keep_first, seg.tile_size, Dv, sigmoid_bias,
+             v_div)
         if Tp >= T:
             return out
         q1, out, T = q1[Tp:], out[Tp:], T - Tp

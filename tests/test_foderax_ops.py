@@ -20,7 +20,7 @@ from lumen.ops.moe import route_groups
 from lumen.ops.norm import depth_mix_norm
 from lumen.ops.recurrent import min_gru_scan
 from lumen.ops.rope import interleaved_inv_freq, rotary_write
-from lumen.ops.segments import SegBatch, tile_list
+from lumen.ops.segments import TILE_ROWS, SegBatch, tile_list
 
 
 # ---- start of the stream, soft cap ------------------------------------------------------------------
@@ -188,6 +188,19 @@ def test_min_gru_candidate_is_continuous_at_zero(device, dtype):
 # ---- attention whose weights are sigmoids --------------------------------------------------------------
 SPANS = [(0, 0, 19), (1, 130, 1), (2, 60, 37), (0, 19, 1), (1, 131, 2), (2, 97, 1), (2, 98, 1)]
 LENS = [20, 133, 99]
+# prompt portions first (one of them longer than a tile), decoded rows after them: the layout of an
+# engine step, with the tile list that sends the portions to the matrix-core kernel
+SPANS_TILED = [(0, 0, 19), (2, 60, 37), (1, 3, 129), (1, 132, 1), (0, 19, 1), (2, 97, 1)]
+
+
+def step_segments(tiled, tb, device):
+    if not tiled:
+        return segments(SPANS, tb, device), SPANS
+    seg = segments(SPANS_TILED, tb, device)
+    cu = seg.cu.tolist()
+    seg.q_tiles = torch.tensor(tile_list(cu, 3), dtype=torch.int32, device=device).view(-1, 2)
+    seg.tile_rows, seg.tile_size = cu[3], TILE_ROWS
+    return seg, SPANS_TILED
 
 
 def dense_sigmoid_attention(q, k, v, pos_q, hg, scale, pb):
@@ -201,15 +214,17 @@ def dense_sigmoid_attention(q, k, v, pos_q, hg, scale, pb):
 
 @pytest.mark.parametrize("device,dtype", CASES)
 @pytest.mark.parametrize("H,G,D,Dv,bs", [(6, 1, 24, 40, 8), (3, 3, 10, 14, 16), (4, 2, 32, 16, 8),
-                                         (16, 4, 128, 128, 16), (2, 2, 96, 192, 16)])
-def test_sigmoid_weight_attention(device, dtype, H, G, D, Dv, bs):
+                                         (16, 4, 128, 128, 16), (2, 2, 96, 192, 16),
+                                         (6, 2, 64, 64, 8), (2, 1, 48, 96, 16)])
+@pytest.mark.parametrize("tiled", [False, True])
+def test_sigmoid_weight_attention(device, dtype, H, G, D, Dv, bs, tiled):
     ks = [rnd(n, G * D, seed=20 + i, dtype=dtype) for i, n in enumerate(LENS)]
     vs = [rnd(n, G * Dv, seed=30 + i, dtype=dtype) for i, n in enumerate(LENS)]
     kc, tb = paged(ks, bs, 40, G * D, dtype, device, 1)
     vc, _ = paged(vs, bs, 40, G * Dv, dtype, device, 1)
-    seg = segments(SPANS, tb, device)
+    seg, SPANS = step_segments(tiled, tb, device)
     T = seg.T
-    q = rnd(T, H * D + 3, seed=40, dtype=dtype, device=device)[:, :H * D].view(T, H, D)
+    q = rnd(T, H * D + 8, seed=40, dtype=dtype, device=device)[:, :H * D].view(T, H, D)
     pb = rnd(H, seed=41, device=device) - 2.0
     out = torch.zeros(T, H, Dv, dtype=dtype, device=device)
     row_attention(q, None, kc.view(40, bs, G, D), vc.view(40, bs, G, Dv), Dv, out, seg, H, G,
@@ -266,8 +281,10 @@ def test_sigmoid_weights_are_not_normalised(device, dtype, far):
 # ---- several score maps over shared values ------------------------------------------------------------
 @pytest.mark.parametrize("device,dtype", CASES)
 @pytest.mark.parametrize("H,G,D,Dv,bs", [(4, 2, 16, 24, 8), (3, 1, 6, 10, 16), (8, 2, 64, 64, 16),
-                                         (2, 2, 128, 256, 16), (3, 1, 48, 96, 8)])
-def test_two_maps_share_values(device, dtype, H, G, D, Dv, bs):
+                                         (2, 2, 128, 256, 16), (3, 1, 48, 96, 8), (4, 1, 32, 64, 16),
+                                         (6, 3, 96, 192, 16)])
+@pytest.mark.parametrize("tiled", [False, True])
+def test_two_maps_share_values(device, dtype, H, G, D, Dv, bs, tiled):
     """2 H query heads on 2 G key heads over G value heads (v_div = 2), laid out [key head][map]
     [head of the group]: every map is a softmax attention of its own over the same values."""
     rep = H // G
@@ -275,7 +292,7 @@ def test_two_maps_share_values(device, dtype, H, G, D, Dv, bs):
     vs = [rnd(n, G * Dv, seed=30 + i, dtype=dtype) for i, n in enumerate(LENS)]
     kc, tb = paged(ks, bs, 40, 2 * G * D, dtype, device, 1)
     vc, _ = paged(vs, bs, 40, G * Dv, dtype, device, 1)
-    seg = segments(SPANS, tb, device)
+    seg, SPANS = step_segments(tiled, tb, device)
     T = seg.T
     q = rnd(T, 2 * H, D, seed=40, dtype=dtype, device=device, scale=2.0)
     out = torch.zeros(T, 2 * H, Dv, dtype=dtype, device=device)
